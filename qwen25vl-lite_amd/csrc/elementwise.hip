@@ -1,0 +1,189 @@
+// Row-wise kernels of the decoder step: embedding gather, residual add + RMSNorm,
+// rotation + cache write, SwiGLU.  Each works for float32 and bfloat16 storage and any
+// row width; all arithmetic is float32.
+#include "common.h"
+
+// ---------------------------------------------------------------------------------------
+// Embedding gather: out[n, :] = float32(table[ids[n], :])       (reference text.py:213)
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ void embed_gather_kernel(const int* __restrict__ ids, const T* __restrict__ table,
+                                    float* __restrict__ out, int H, int V) {
+  const int n = blockIdx.x;
+  int id = ids[n];
+  id = id < 0 ? 0 : (id >= V ? V - 1 : id);  // ids are validated on the host; never read outside the table
+  const T* row = table + (size_t)id * H;
+  float* o = out + (size_t)n * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = ldf<T>(row + i);
+}
+
+extern "C" int qvl_embed_gather(const void* ids, const void* table, void* out, int N, int H, int V, int dtype,
+                                hipStream_t stream) {
+  if (N <= 0) return QVL_OK;
+  if (H <= 0 || V <= 0) return QVL_ERR_SHAPE;
+  if (dtype == 0)
+    hipLaunchKernelGGL(embed_gather_kernel<float>, dim3(N), dim3(256), 0, stream, (const int*)ids,
+                       (const float*)table, (float*)out, H, V);
+  else if (dtype == 1)
+    hipLaunchKernelGGL(embed_gather_kernel<bf16_t>, dim3(N), dim3(256), 0, stream, (const int*)ids,
+                       (const bf16_t*)table, (float*)out, H, V);
+  else
+    return QVL_ERR_DTYPE;
+  return qvl_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------
+// Residual add + RMSNorm  (reference layers.py:27-31, text.py:196-205)
+//   v = h[row] + delta[row]            (delta optional; the sum is float32)
+//   h[row] = v                         (unless `rows` selects rows: then h is left alone)
+//   out[m] = v * (1/sqrt(mean(v^2) + eps)) * w
+// One block per row; the reduction order depends on H only, so a row's result does not
+// depend on what else is in the batch.
+// ---------------------------------------------------------------------------------------
+template <typename TD, typename TO>
+__global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__ delta, const float* __restrict__ w,
+                                   TO* __restrict__ out, const int* __restrict__ rows, int H, float eps) {
+  __shared__ float red[17];
+  const int m = blockIdx.x;
+  const int row = rows ? rows[m] : m;
+  float* hr = h + (size_t)row * H;
+  const TD* dr = delta ? delta + (size_t)row * H : nullptr;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float v = hr[i];
+    if (dr) v += ldf<TD>(dr + i);
+    ss += v * v;
+    if (dr && !rows) hr[i] = v;
+  }
+  const float total = block_sum(ss, red);
+  const float rs = 1.0f / sqrtf(total / (float)H + eps);
+  TO* o = out + (size_t)m * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float v = hr[i];
+    if (dr && rows) v += ldf<TD>(dr + i);
+    stf<TO>(o + i, (v * rs) * w[i]);
+  }
+}
+
+extern "C" int qvl_add_rmsnorm(void* h, const void* delta, const void* w, void* out, const void* rows, int M, int H,
+                               float eps, int dtype, hipStream_t stream) {
+  if (M <= 0) return QVL_OK;
+  if (H <= 0) return QVL_ERR_SHAPE;
+  const int threads = H >= 2048 ? 512 : 256;
+  if (dtype == 0)
+    hipLaunchKernelGGL((add_rmsnorm_kernel<float, float>), dim3(M), dim3(threads), 0, stream, (float*)h,
+                       (const float*)delta, (const float*)w, (float*)out, (const int*)rows, H, eps);
+  else if (dtype == 1)
+    hipLaunchKernelGGL((add_rmsnorm_kernel<bf16_t, bf16_t>), dim3(M), dim3(threads), 0, stream, (float*)h,
+                       (const bf16_t*)delta, (const float*)w, (bf16_t*)out, (const int*)rows, H, eps);
+  else
+    return QVL_ERR_DTYPE;
+  return qvl_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------
+// Rotation + cache write  (reference rope.py:48-96, cache.py:440-460)
+// x[n] holds nq query heads, then nkv key heads, then nkv value heads, each hd wide.
+// For frequency f < rot_half the angle is float32(pos[freq_row[f]][n]) * inv_freq[f]; the pair
+// is (f, f + rot_half):  out[f] = x[f] c - x[f+rot_half] s,  out[f+rot_half] = x[f+rot_half] c + x[f] s.
+// Channels from 2*rot_half on pass unrotated.  Queries go to q_out; keys (rotated) and values
+// go into the page slot of the token: K as [page][kv head][slot][hd], V as [page][kv head][hd][slot].
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ void rope_kv_write_kernel(const T* __restrict__ x, int x_stride, const float* __restrict__ bias,
+                                     const int* __restrict__ pos, int pos_stride,
+                                     const float* __restrict__ inv_freq, const int* __restrict__ freq_row,
+                                     const int* __restrict__ slot, T* __restrict__ q_out, T* __restrict__ kc,
+                                     T* __restrict__ vc, int nq, int nkv, int hd, int rot_half, int ps) {
+  const int n = blockIdx.x;
+  const int hh = blockIdx.y;
+  const T* src = x + (size_t)n * x_stride + (size_t)hh * hd;
+  const float* b = bias ? bias + (size_t)hh * hd : nullptr;
+  if (hh >= nq + nkv) {  // value head: copy
+    const int s = slot[n];
+    if (s < 0) return;
+    const int kvh = hh - nq - nkv;
+    const size_t page = (size_t)(s / ps), off = (size_t)(s % ps);
+    T* dst = vc + ((page * nkv + kvh) * hd) * ps + off;
+    for (int d = threadIdx.x; d < hd; d += blockDim.x) {
+      float v = ldf<T>(src + d) + (b ? b[d] : 0.f);
+      stf<T>(dst + (size_t)d * ps, v);
+    }
+    return;
+  }
+  T* dst;
+  if (hh < nq) {
+    dst = q_out + ((size_t)n * nq + hh) * hd;
+  } else {
+    const int s = slot[n];
+    if (s < 0) return;
+    const int kvh = hh - nq;
+    const size_t page = (size_t)(s / ps), off = (size_t)(s % ps);
+    dst = kc + ((page * nkv + kvh) * ps + off) * hd;
+  }
+  for (int f = threadIdx.x; f < rot_half; f += blockDim.x) {
+    float x1 = ldf<T>(src + f) + (b ? b[f] : 0.f);
+    float x2 = ldf<T>(src + f + rot_half) + (b ? b[f + rot_half] : 0.f);
+    const int row = freq_row[f];
+    float c = 1.f, s = 0.f;
+    if (row >= 0) {
+      const float ang = (float)pos[(size_t)row * pos_stride + n] * inv_freq[f];
+      sincosf(ang, &s, &c);
+    }
+    stf<T>(dst + f, x1 * c - x2 * s);
+    stf<T>(dst + f + rot_half, x2 * c + x1 * s);
+  }
+  for (int d = 2 * rot_half + threadIdx.x; d < hd; d += blockDim.x)
+    stf<T>(dst + d, ldf<T>(src + d) + (b ? b[d] : 0.f));
+}
+
+extern "C" int qvl_rope_kv_write(const void* x, int x_stride, const void* bias, const void* pos, int pos_stride,
+                                 const void* inv_freq, const void* freq_row, const void* slot, void* q_out, void* kc,
+                                 void* vc, int N, int nq, int nkv, int hd, int rot_half, int ps, int dtype,
+                                 hipStream_t stream) {
+  if (N <= 0) return QVL_OK;
+  if (nq < 0 || nkv < 0 || nq + nkv == 0 || hd <= 0 || rot_half < 0 || 2 * rot_half > hd || ps <= 0)
+    return QVL_ERR_SHAPE;
+  if (x_stride < (nq + 2 * nkv) * hd) return QVL_ERR_SHAPE;
+  if (nq + 2 * nkv > 65535) return QVL_ERR_LIMIT;
+  const dim3 grid(N, nq + 2 * nkv);
+  if (dtype == 0)
+    hipLaunchKernelGGL(rope_kv_write_kernel<float>, grid, dim3(64), 0, stream, (const float*)x, x_stride,
+                       (const float*)bias, (const int*)pos, pos_stride, (const float*)inv_freq, (const int*)freq_row,
+                       (const int*)slot, (float*)q_out, (float*)kc, (float*)vc, nq, nkv, hd, rot_half, ps);
+  else if (dtype == 1)
+    hipLaunchKernelGGL(rope_kv_write_kernel<bf16_t>, grid, dim3(64), 0, stream, (const bf16_t*)x, x_stride,
+                       (const float*)bias, (const int*)pos, pos_stride, (const float*)inv_freq, (const int*)freq_row,
+                       (const int*)slot, (bf16_t*)q_out, (bf16_t*)kc, (bf16_t*)vc, nq, nkv, hd, rot_half, ps);
+  else
+    return QVL_ERR_DTYPE;
+  return qvl_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------
+// SwiGLU: out[n, i] = silu(x[n, i]) * x[n, I + i],  silu(z) = z / (1 + exp(-z))
+// (reference text.py:66)
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ x, T* __restrict__ out, int I) {
+  const int n = blockIdx.y;
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= I) return;
+  const T* row = x + (size_t)n * 2 * I;
+  const float g = ldf<T>(row + i), u = ldf<T>(row + I + i);
+  stf<T>(out + (size_t)n * I + i, (g / (1.0f + expf(-g))) * u);
+}
+
+extern "C" int qvl_swiglu(const void* x, void* out, int N, int I, int dtype, hipStream_t stream) {
+  if (N <= 0) return QVL_OK;
+  if (I <= 0) return QVL_ERR_SHAPE;
+  if (N > 65535) return QVL_ERR_LIMIT;
+  const dim3 grid((I + 255) / 256, N);
+  if (dtype == 0)
+    hipLaunchKernelGGL(swiglu_kernel<float>, grid, dim3(256), 0, stream, (const float*)x, (float*)out, I);
+  else if (dtype == 1)
+    hipLaunchKernelGGL(swiglu_kernel<bf16_t>, grid, dim3(256), 0, stream, (const bf16_t*)x, (bf16_t*)out, I);
+  else
+    return QVL_ERR_DTYPE;
+  return qvl_launch_status();
+}

@@ -1,0 +1,88 @@
+"""The step function: runs a batch of (request, its next tokens) through the model from the
+cache and returns the logits at the wanted places.
+
+Reference counterpart: ``ModelRunner`` (reference src/qwen25vl_lite/engine.py:204-486), which
+runs a prompt portion of one request or single tokens of several, never both.  Here both
+share one batch: only the tokens brought are run, as one flat batch, against the keys and
+values earlier steps left in the pages.
+"""
+
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence
+
+import torch
+
+from ..cache import CacheManager, KVStorage
+from ..config.engine_config import EngineConfig
+from ..models.decoder import DecoderModel
+from .batch import StepEntry, build_step
+
+__all__ = ["ModelRunner"]
+
+
+class ModelRunner:
+    """Owns the cache (manager and tensors) and the per-request state, and steps the model."""
+
+    def __init__(self, model: DecoderModel, engine_cfg: EngineConfig, *, max_prefix_nodes: int = 4096):
+        if model.device.type != "cuda":
+            raise RuntimeError("the model runs on the GPU only; build it with device='cuda:0'")
+        if model.dtype != engine_cfg.dtype:
+            raise ValueError(f"the model holds {model.dtype} weights but the engine is set to {engine_cfg.dtype}")
+        self.model = model
+        self.ecfg = engine_cfg
+        self.device = model.device
+        self.dtype = model.dtype
+        self.vocab_size = model.spec.vocab_size
+        self.eos_token_id = model.spec.eos_token_id
+        groups = model.cache_groups()
+        self.cache = CacheManager(groups, engine_cfg.num_blocks, engine_cfg.block_size, engine_cfg.max_num_seqs,
+                                  enable_prefix_cache=engine_cfg.enable_prefix_cache,
+                                  max_prefix_nodes=max_prefix_nodes)
+        self.storage = KVStorage(groups, engine_cfg.num_blocks, engine_cfg.block_size, self.dtype, self.device)
+        self.states: List[Optional[torch.Tensor]] = [
+            None if need is None else torch.zeros((engine_cfg.max_num_seqs, *need.shape), dtype=need.dtype,
+                                                  device=self.device)
+            for need in model.entry_state
+        ]
+        self.slots = model.make_slots(self.storage, self.states)
+        self.steps = 0
+
+    # ------------------------------------------------------------------ requests
+    def admit(self, req_id) -> int:
+        return self.cache.admit(req_id)
+
+    def release(self, req_id) -> None:
+        self.cache.release(req_id)
+
+    def _clear_state(self, entries: Sequence[StepEntry]) -> None:
+        for e in entries:
+            if self.cache.take_fresh(e.req_id):
+                slot = self.cache.slot_of(e.req_id)
+                for state in self.states:
+                    if state is not None:
+                        state[slot].zero_()
+
+    # ------------------------------------------------------------------ the step
+    @torch.no_grad()
+    def execute(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Run one step.  Pages for the new tokens are reserved here if the caller has not done
+        so (:class:`~qwen25vl_lite_amd.cache.OutOfPages` if they cannot be).  Returns float32 logits
+        ``[wanted, vocab]`` in the order of the entries and of each entry's ``want``."""
+        for e in entries:
+            self.cache.reserve(e.req_id, e.start + len(e.tokens))
+        self._clear_state(entries)
+        with torch.cuda.device(self.device):
+            step = build_step(entries, self.cache, self.model.spec.position_rows, self.dtype, self.device,
+                              self.vocab_size)
+            logits = self.model.forward(step, self.slots)
+        for e in entries:
+            self.cache.commit(e.req_id, e.start + len(e.tokens))
+        self.steps += 1
+        return logits
+
+    def sample(self, logits: torch.Tensor, params: Sequence, prev_ids: Sequence[Sequence[int]],
+               steps: Sequence[int]) -> List[int]:
+        """One token per logits row, on the device (see :mod:`qwen25vl_lite_amd.sampling`)."""
+        from ..sampling.sampler import sample_rows
+        return sample_rows(logits, params, prev_ids, steps)

@@ -1,0 +1,145 @@
+"""A decoder built from a :class:`ModelSpec`: embedding, the run list of layers, the final
+norm and the output head (reference src/qwen25vl_lite/text.py:209-279, model.py:84-86, 200-202).
+"""
+
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Tuple
+
+import torch
+
+from ..cache.manager import CacheGroupSpec
+from ..ops import kernels
+from ..ops.linear import linear
+from ..parts.base import (Block, CacheNeed, LayerSlot, Mixer, ParamSpec, Part, ResidualStream, StateNeed,
+                          StepContext, build_part)
+from .spec import ModelSpec
+
+__all__ = ["DecoderModel"]
+
+
+def _collect(part: Part, prefix: str, out: Dict[str, Tuple[Part, str, ParamSpec]]) -> None:
+    for local, spec in part.param_specs().items():
+        out[prefix + local] = (part, local, spec)
+    for name, sub in part.sub_parts().items():
+        _collect(sub, f"{prefix}{name}.", out)
+
+
+def _mixer_of(block: Block) -> Optional[Mixer]:
+    for sub in block.sub_parts().values():
+        if isinstance(sub, Mixer):
+            return sub
+    return None
+
+
+class DecoderModel:
+    """Holds the parts and runs a step over them.  Tensors arrive through :meth:`load_part`."""
+
+    def __init__(self, spec: ModelSpec, dtype: torch.dtype, device):
+        self.spec = spec
+        self.dtype = dtype
+        self.device = torch.device(device)
+        self.blocks: List[Block] = [build_part("block", ls.block, dtype, self.device) for ls in spec.layers]
+        self.final_norm = build_part("norm", spec.final_norm, dtype, self.device)
+        self.embed: Optional[torch.Tensor] = None
+        self.head: Optional[torch.Tensor] = None
+
+        # the run list: which cache layer and state each entry owns
+        self.group_needs: List[CacheNeed] = []
+        self.group_layers: List[int] = []
+        self.entry_group: List[Optional[int]] = []
+        self.entry_cache_layer: List[Optional[int]] = []
+        self.entry_writes: List[bool] = []
+        self.entry_state: List[Optional[StateNeed]] = []
+        for i, entry in enumerate(spec.run):
+            if not 0 <= entry.layer < len(self.blocks):
+                raise ValueError(f"run entry {i} names layer {entry.layer}, which does not exist")
+            mixer = _mixer_of(self.blocks[entry.layer])
+            need = mixer.cache_need() if mixer is not None else None
+            self.entry_state.append(mixer.state_need() if mixer is not None else None)
+            if need is None:
+                if entry.cache_from is not None:
+                    raise ValueError(f"run entry {i} reads a cache but its mixer keeps none")
+                self.entry_group.append(None)
+                self.entry_cache_layer.append(None)
+                self.entry_writes.append(False)
+                continue
+            if entry.cache_from is not None:
+                src = entry.cache_from
+                if not 0 <= src < i or self.entry_group[src] is None or not self.entry_writes[src]:
+                    raise ValueError(f"run entry {i} must read the cache of an earlier entry that writes one")
+                if self.group_needs[self.entry_group[src]] != need:
+                    raise ValueError(f"run entry {i} reads the cache of entry {src}, whose shape or window differs")
+                self.entry_group.append(self.entry_group[src])
+                self.entry_cache_layer.append(self.entry_cache_layer[src])
+                self.entry_writes.append(False)
+                continue
+            if need not in self.group_needs:
+                self.group_needs.append(need)
+                self.group_layers.append(0)
+            g = self.group_needs.index(need)
+            self.entry_group.append(g)
+            self.entry_cache_layer.append(self.group_layers[g])
+            self.entry_writes.append(True)
+            self.group_layers[g] += 1
+
+        self.params: Dict[str, Tuple[Optional[Part], str, ParamSpec]] = {}
+        self.params[spec.embed_name] = (None, "embed", ParamSpec((spec.vocab_size, spec.hidden_size), "table"))
+        for ls, block in zip(spec.layers, self.blocks):
+            _collect(block, ls.prefix, self.params)
+        _collect(self.final_norm, spec.final_norm_prefix, self.params)
+        self.params[spec.head_name] = (None, "head", ParamSpec((spec.vocab_size, spec.hidden_size), "matrix"))
+
+    # ------------------------------------------------------------------ structure
+    def cache_groups(self) -> List[CacheGroupSpec]:
+        return [CacheGroupSpec(need, n) for need, n in zip(self.group_needs, self.group_layers)]
+
+    def expected_tensors(self) -> Dict[str, ParamSpec]:
+        """Canonical tensor name -> what is expected under it."""
+        return {name: spec for name, (_, _, spec) in self.params.items()}
+
+    def part_groups(self) -> List[Tuple[Optional[Part], Dict[str, str]]]:
+        """Tensors grouped by the part that takes them: ``(part, {local: canonical})``."""
+        groups: Dict[int, Tuple[Optional[Part], Dict[str, str]]] = {}
+        for name, (part, local, _) in self.params.items():
+            key = id(part) if part is not None else hash(name)
+            groups.setdefault(key, (part, {}))[1][local] = name
+        return list(groups.values())
+
+    def load_part(self, part: Optional[Part], tensors: Dict[str, torch.Tensor]) -> None:
+        if part is not None:
+            part.load(tensors)
+        elif "embed" in tensors:
+            self.embed = tensors["embed"]
+        elif "head" in tensors:
+            self.head = tensors["head"]
+
+    def tie_head(self) -> None:
+        self.head = self.embed
+
+    def make_slots(self, storage, state_tensors: List[Optional[torch.Tensor]]) -> List[LayerSlot]:
+        slots = []
+        for i in range(len(self.spec.run)):
+            g, layer = self.entry_group[i], self.entry_cache_layer[i]
+            slots.append(LayerSlot(
+                group=g,
+                k_cache=storage.k[g][layer] if g is not None else None,
+                v_cache=storage.v[g][layer] if g is not None else None,
+                writes=self.entry_writes[i],
+                state=state_tensors[i],
+            ))
+        return slots
+
+    # ------------------------------------------------------------------ the step
+    def forward(self, step: StepContext, slots: List[LayerSlot]) -> torch.Tensor:
+        """Run the step's tokens through the run list; float32 logits ``[M, vocab]`` at
+        ``step.logit_rows``."""
+        if self.embed is None or self.head is None:
+            raise RuntimeError("the model has no weights yet")
+        stream = ResidualStream(kernels.embed_gather(step.token_ids, self.embed))
+        for entry, slot in zip(self.spec.run, slots):
+            stream = self.blocks[entry.layer].forward(stream, step, slot)
+        if step.logit_rows.shape[0] == 0:
+            return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)
+        x = self.final_norm.forward(stream, rows=step.logit_rows)
+        return linear(x, self.head, out_dtype=torch.float32)

@@ -1,0 +1,1 @@
+"""Hand-written HIP kernels for gfx950 and their Python entry points."""

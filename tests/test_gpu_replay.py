@@ -1,0 +1,107 @@
+"""The engine against the plain implementation, replayed in every way of cutting and batching."""
+
+import pytest
+import torch
+
+from plain_model import plain_model_logits
+from replay_util import (mixed_trace, portion_trace, random_tokens, round64, run_steps, tail_trace, whole_trace)
+
+pytestmark = pytest.mark.gpu
+
+LENGTHS = {"A": [5, 17, 33, 70], "B": [1, 9, 40, 64, 97], "C": [3, 48, 81, 130]}
+VOCAB = {"A": 256, "B": 509, "C": 300}
+
+
+def _requests(name):
+    return {f"r{i}": random_tokens(n, VOCAB[name], 100 * ord(name) + i) for i, n in enumerate(LENGTHS[name])}
+
+
+def _reference(model_dir, requests):
+    return {rid: plain_model_logits(model_dir, toks) for rid, toks in requests.items()}
+
+
+def _compare(got, ref, dtype, what):
+    worst = 0.0
+    for (rid, pos), row in got.items():
+        want = ref[rid][pos]
+        if dtype == "float32":
+            # the reference's own criterion (reference tests/test_chunked_prefill.py:81)
+            ok = torch.allclose(row, want, atol=1e-4, rtol=1e-3)
+            err = (row - want).abs().max().item()
+        else:
+            # bfloat16: worst error against the largest logit, as the reference checks its fused
+            # kernel (reference src/qwen25vl_lite/paged_attn_triton.py:253)
+            err = ((row - want).abs().max() / want.abs().max()).item()
+            ok = err < 2e-2
+        worst = max(worst, err)
+        assert ok, f"{what}: request {rid} position {pos}: error {err:.3e}"
+    return worst
+
+
+def _replayer(model_dir, dtype, max_tokens):
+    from qwen25vl_lite_amd.engine.replay import Replayer
+    return Replayer(model_dir, dtype, max_tokens)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_replay_every_way(model_dirs, name, dtype):
+    d = model_dirs[name]
+    requests = _requests(name)
+    ref = _reference(d, requests)
+    total = sum(len(t) for t in requests.values())
+
+    rp = _replayer(d, dtype, round64(max(LENGTHS[name])))
+    got = run_steps(rp, whole_trace(requests))
+    assert len(got) == total
+    print(name, dtype, "whole", _compare(got, ref, dtype, "whole"))
+    assert rp.runner.cache.pages_in_use() == [0] * len(rp.runner.cache.groups)
+
+    got = run_steps(rp, tail_trace(requests))
+    assert len(got) == total
+    print(name, dtype, "tail", _compare(got, ref, dtype, "tail"))
+
+    got = run_steps(rp, portion_trace(requests))
+    assert len(got) == total
+    print(name, dtype, "portions", _compare(got, ref, dtype, "portions"))
+    rp.runner.cache.check()
+
+    steps, peak = mixed_trace(requests, seed=7)
+    rp = _replayer(d, dtype, peak)
+    got = run_steps(rp, steps)
+    assert len(got) == total
+    print(name, dtype, "mixed", _compare(got, ref, dtype, "mixed"), "pool tokens", peak)
+    rp.runner.cache.check()
+    assert rp.runner.cache.pages_in_use() == [0] * len(rp.runner.cache.groups)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_explicit_position_rows(model_dirs, dtype):
+    """Distinct t/h/w rows for a 4x4 block inside the prompt, then text with a rope delta
+    (reference rope.py:137-235 builds such rows for an image grid)."""
+    d = model_dirs["B"]
+    toks = random_tokens(40, VOCAB["B"], 5)
+    t_row, h_row, w_row = [], [], []
+    for p in range(6):
+        t_row.append(p), h_row.append(p), w_row.append(p)
+    for i in range(16):  # a 4x4 grid starting at position 6
+        t_row.append(6), h_row.append(6 + i // 4), w_row.append(6 + i % 4)
+    nxt = 10
+    delta = nxt - 22
+    for p in range(22, 40):
+        t_row.append(p + delta), h_row.append(p + delta), w_row.append(p + delta)
+    pos = [t_row, h_row, w_row]
+    ref = plain_model_logits(d, toks, torch.tensor(pos))
+    rp = _replayer(d, dtype, 64)
+    # the prompt (with explicit rows) in two portions, the text after it by the delta rule
+    steps = [
+        {"step": 0, "entries": [{"id": "x", "tokens": toks[:9], "positions": [r[:9] for r in pos],
+                                 "want": list(range(9))}], "end": []},
+        {"step": 1, "entries": [{"id": "x", "tokens": toks[9:22], "positions": [r[9:22] for r in pos],
+                                 "want": list(range(13)), "rope_delta": delta}], "end": []},
+        {"step": 2, "entries": [{"id": "x", "tokens": toks[22:30], "want": list(range(8))}], "end": []},
+    ] + [{"step": 3 + i, "entries": [{"id": "x", "tokens": [toks[30 + i]], "want": [0]}], "end": []}
+         for i in range(10)]
+    got = run_steps(rp, steps)
+    assert len(got) == 40
+    _compare(got, {"x": ref}, dtype, "explicit rows")
