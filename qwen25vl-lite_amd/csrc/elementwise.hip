@@ -66,19 +66,22 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__
 }
 
 extern "C" int qvl_add_rmsnorm(void* h, const void* delta, const void* w, void* out, const void* rows, int M, int H,
-                               float eps, int dtype, hipStream_t stream) {
+                               float eps, int delta_dtype, int out_dtype, hipStream_t stream) {
   if (M <= 0) return QVL_OK;
   if (H <= 0) return QVL_ERR_SHAPE;
   const int threads = H >= 2048 ? 512 : 256;
-  if (dtype == 0)
-    hipLaunchKernelGGL((add_rmsnorm_kernel<float, float>), dim3(M), dim3(threads), 0, stream, (float*)h,
-                       (const float*)delta, (const float*)w, (float*)out, (const int*)rows, H, eps);
-  else if (dtype == 1)
-    hipLaunchKernelGGL((add_rmsnorm_kernel<bf16_t, bf16_t>), dim3(M), dim3(threads), 0, stream, (float*)h,
-                       (const bf16_t*)delta, (const float*)w, (bf16_t*)out, (const int*)rows, H, eps);
-  else
-    return QVL_ERR_DTYPE;
-  return qvl_launch_status();
+#define QVL_NORM_CASE(DD, OD, TD, TO)                                                                              \
+  if (delta_dtype == DD && out_dtype == OD) {                                                                      \
+    hipLaunchKernelGGL((add_rmsnorm_kernel<TD, TO>), dim3(M), dim3(threads), 0, stream, (float*)h,                 \
+                       (const TD*)delta, (const float*)w, (TO*)out, (const int*)rows, H, eps);                     \
+    return qvl_launch_status();                                                                                    \
+  }
+  QVL_NORM_CASE(0, 0, float, float)
+  QVL_NORM_CASE(0, 1, float, bf16_t)
+  QVL_NORM_CASE(1, 1, bf16_t, bf16_t)
+  QVL_NORM_CASE(1, 0, bf16_t, float)
+#undef QVL_NORM_CASE
+  return QVL_ERR_DTYPE;
 }
 
 // ---------------------------------------------------------------------------------------
@@ -89,15 +92,15 @@ extern "C" int qvl_add_rmsnorm(void* h, const void* delta, const void* w, void* 
 // Channels from 2*rot_half on pass unrotated.  Queries go to q_out; keys (rotated) and values
 // go into the page slot of the token: K as [page][kv head][slot][hd], V as [page][kv head][hd][slot].
 // ---------------------------------------------------------------------------------------
-template <typename T>
-__global__ void rope_kv_write_kernel(const T* __restrict__ x, int x_stride, const float* __restrict__ bias,
+template <typename TI, typename T>
+__global__ void rope_kv_write_kernel(const TI* __restrict__ x, int x_stride, const float* __restrict__ bias,
                                      const int* __restrict__ pos, int pos_stride,
                                      const float* __restrict__ inv_freq, const int* __restrict__ freq_row,
                                      const int* __restrict__ slot, T* __restrict__ q_out, T* __restrict__ kc,
                                      T* __restrict__ vc, int nq, int nkv, int hd, int rot_half, int ps) {
   const int n = blockIdx.x;
   const int hh = blockIdx.y;
-  const T* src = x + (size_t)n * x_stride + (size_t)hh * hd;
+  const TI* src = x + (size_t)n * x_stride + (size_t)hh * hd;
   const float* b = bias ? bias + (size_t)hh * hd : nullptr;
   if (hh >= nq + nkv) {  // value head: copy
     const int s = slot[n];
@@ -106,7 +109,7 @@ __global__ void rope_kv_write_kernel(const T* __restrict__ x, int x_stride, cons
     const size_t page = (size_t)(s / ps), off = (size_t)(s % ps);
     T* dst = vc + ((page * nkv + kvh) * hd) * ps + off;
     for (int d = threadIdx.x; d < hd; d += blockDim.x) {
-      float v = ldf<T>(src + d) + (b ? b[d] : 0.f);
+      float v = ldf<TI>(src + d) + (b ? b[d] : 0.f);
       stf<T>(dst + (size_t)d * ps, v);
     }
     return;
@@ -122,8 +125,8 @@ __global__ void rope_kv_write_kernel(const T* __restrict__ x, int x_stride, cons
     dst = kc + ((page * nkv + kvh) * ps + off) * hd;
   }
   for (int f = threadIdx.x; f < rot_half; f += blockDim.x) {
-    float x1 = ldf<T>(src + f) + (b ? b[f] : 0.f);
-    float x2 = ldf<T>(src + f + rot_half) + (b ? b[f + rot_half] : 0.f);
+    float x1 = ldf<TI>(src + f) + (b ? b[f] : 0.f);
+    float x2 = ldf<TI>(src + f + rot_half) + (b ? b[f + rot_half] : 0.f);
     const int row = freq_row[f];
     float c = 1.f, s = 0.f;
     if (row >= 0) {
@@ -134,30 +137,32 @@ __global__ void rope_kv_write_kernel(const T* __restrict__ x, int x_stride, cons
     stf<T>(dst + f + rot_half, x2 * c + x1 * s);
   }
   for (int d = 2 * rot_half + threadIdx.x; d < hd; d += blockDim.x)
-    stf<T>(dst + d, ldf<T>(src + d) + (b ? b[d] : 0.f));
+    stf<T>(dst + d, ldf<TI>(src + d) + (b ? b[d] : 0.f));
 }
 
 extern "C" int qvl_rope_kv_write(const void* x, int x_stride, const void* bias, const void* pos, int pos_stride,
                                  const void* inv_freq, const void* freq_row, const void* slot, void* q_out, void* kc,
-                                 void* vc, int N, int nq, int nkv, int hd, int rot_half, int ps, int dtype,
-                                 hipStream_t stream) {
+                                 void* vc, int N, int nq, int nkv, int hd, int rot_half, int ps, int in_dtype,
+                                 int dtype, hipStream_t stream) {
   if (N <= 0) return QVL_OK;
   if (nq < 0 || nkv < 0 || nq + nkv == 0 || hd <= 0 || rot_half < 0 || 2 * rot_half > hd || ps <= 0)
     return QVL_ERR_SHAPE;
   if (x_stride < (nq + 2 * nkv) * hd) return QVL_ERR_SHAPE;
   if (nq + 2 * nkv > 65535) return QVL_ERR_LIMIT;
   const dim3 grid(N, nq + 2 * nkv);
-  if (dtype == 0)
-    hipLaunchKernelGGL(rope_kv_write_kernel<float>, grid, dim3(64), 0, stream, (const float*)x, x_stride,
-                       (const float*)bias, (const int*)pos, pos_stride, (const float*)inv_freq, (const int*)freq_row,
-                       (const int*)slot, (float*)q_out, (float*)kc, (float*)vc, nq, nkv, hd, rot_half, ps);
-  else if (dtype == 1)
-    hipLaunchKernelGGL(rope_kv_write_kernel<bf16_t>, grid, dim3(64), 0, stream, (const bf16_t*)x, x_stride,
-                       (const float*)bias, (const int*)pos, pos_stride, (const float*)inv_freq, (const int*)freq_row,
-                       (const int*)slot, (bf16_t*)q_out, (bf16_t*)kc, (bf16_t*)vc, nq, nkv, hd, rot_half, ps);
-  else
-    return QVL_ERR_DTYPE;
-  return qvl_launch_status();
+#define QVL_ROPE_CASE(ID, OD, TI, T)                                                                               \
+  if (in_dtype == ID && dtype == OD) {                                                                             \
+    hipLaunchKernelGGL((rope_kv_write_kernel<TI, T>), grid, dim3(64), 0, stream, (const TI*)x, x_stride,           \
+                       (const float*)bias, (const int*)pos, pos_stride, (const float*)inv_freq,                    \
+                       (const int*)freq_row, (const int*)slot, (T*)q_out, (T*)kc, (T*)vc, nq, nkv, hd, rot_half,   \
+                       ps);                                                                                        \
+    return qvl_launch_status();                                                                                    \
+  }
+  QVL_ROPE_CASE(0, 0, float, float)
+  QVL_ROPE_CASE(0, 1, float, bf16_t)
+  QVL_ROPE_CASE(1, 1, bf16_t, bf16_t)
+#undef QVL_ROPE_CASE
+  return QVL_ERR_DTYPE;
 }
 
 // ---------------------------------------------------------------------------------------

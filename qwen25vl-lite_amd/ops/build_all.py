@@ -13,6 +13,7 @@ LIBRARIES = [
     ("elementwise", {}),
     ("attention_generic", {}),
     ("gemm_f32", {}),
+    ("sample", {}),
 ]
 
 

@@ -102,8 +102,7 @@ def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Te
     _need(weight.dtype == torch.float32 and weight.shape == (width,) and weight.is_contiguous(),
           "norm weight must be float32 [H]")
     if delta is not None:
-        _need(delta.shape == h.shape and delta.is_contiguous() and delta.dtype == out_dtype,
-              "delta must match h's shape and the activation dtype")
+        _need(delta.shape == h.shape and delta.is_contiguous(), "delta must match h's shape")
     m = n
     if rows is not None:
         _need(rows.dtype == torch.int32 and rows.dim() == 1 and rows.is_contiguous(), "rows must be int32 [M]")
@@ -112,17 +111,22 @@ def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Te
         out = torch.empty((m, width), dtype=out_dtype, device=h.device)
     _need(out.shape == (m, width) and out.dtype == out_dtype and out.is_contiguous(), "out must be [M, H]")
     fn = _fn("elementwise", "qvl_add_rmsnorm",
-             [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_ptr])
+             [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr])
     _check(fn(_ptr(h), _ptr(delta), _ptr(weight), _ptr(out), _ptr(rows), m, width, float(eps),
-              dtype_code(out_dtype), _stream()), "add_rmsnorm")
+              dtype_code(delta.dtype if delta is not None else out_dtype), dtype_code(out_dtype), _stream()),
+           "add_rmsnorm")
     return out
 
 
 def rope_kv_write(x: torch.Tensor, bias: Optional[torch.Tensor], positions: torch.Tensor, inv_freq: torch.Tensor,
                   freq_row: torch.Tensor, slots: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
                   v_cache: Optional[torch.Tensor], num_q_heads: int, num_kv_heads: int, head_dim: int,
-                  page_size: int, q_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                  page_size: int, out_dtype: Optional[torch.dtype] = None,
+                  q_out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Rotate queries and keys, write keys and values into their page slots, return queries.
+
+    ``x`` may be float32 while queries and the cache are bfloat16 (``out_dtype``): the bias is
+    added and the rotation done in float32 and each value is rounded once.
 
     ``x`` is ``[N, (nq + 2 nkv) hd]``: query heads, key heads, value heads.  ``positions`` is
     int32 ``[rows, N]``; ``freq_row[f]`` names the row that frequency ``f`` uses (-1: none).
@@ -134,6 +138,7 @@ def rope_kv_write(x: torch.Tensor, bias: Optional[torch.Tensor], positions: torc
     nq, nkv, hd = int(num_q_heads), int(num_kv_heads), int(head_dim)
     cols = (nq + 2 * nkv) * hd
     _need(x.dim() == 2 and x.shape[1] == cols and x.stride(1) == 1, "x must be [N, (nq + 2 nkv) hd]")
+    odt = out_dtype or x.dtype
     rot_half = inv_freq.shape[0]
     _need(inv_freq.dtype == torch.float32 and inv_freq.is_contiguous() and 2 * rot_half <= hd,
           "inv_freq must be float32 [rot/2] with rot <= head_dim")
@@ -147,21 +152,21 @@ def rope_kv_write(x: torch.Tensor, bias: Optional[torch.Tensor], positions: torc
     if nkv:
         _need(slots is not None and slots.dtype == torch.int32 and slots.shape == (n,) and slots.is_contiguous(),
               "slots must be int32 [N]")
-        _need(k_cache is not None and v_cache is not None and k_cache.dtype == x.dtype and v_cache.dtype == x.dtype,
+        _need(k_cache is not None and v_cache is not None and k_cache.dtype == odt and v_cache.dtype == odt,
               "the cache must have the activation dtype")
         _need(k_cache.is_contiguous() and k_cache.dim() == 4 and tuple(k_cache.shape[1:]) == (nkv, page_size, hd),
               "k_cache must be [pages, nkv, page_size, hd]")
         _need(v_cache.is_contiguous() and v_cache.dim() == 4 and tuple(v_cache.shape[1:]) == (nkv, hd, page_size)
               and v_cache.shape[0] == k_cache.shape[0], "v_cache must be [pages, nkv, hd, page_size]")
     if q_out is None:
-        q_out = torch.empty((n, nq * hd), dtype=x.dtype, device=x.device)
-    _need(q_out.shape == (n, nq * hd) and q_out.dtype == x.dtype and q_out.is_contiguous(), "q_out must be [N, nq hd]")
+        q_out = torch.empty((n, nq * hd), dtype=odt, device=x.device)
+    _need(q_out.shape == (n, nq * hd) and q_out.dtype == odt and q_out.is_contiguous(), "q_out must be [N, nq hd]")
     fn = _fn("elementwise", "qvl_rope_kv_write",
              [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
-              _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+              _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
     _check(fn(_ptr(x), x.stride(0), _ptr(bias), _ptr(positions), positions.stride(0), _ptr(inv_freq),
               _ptr(freq_row), _ptr(slots), _ptr(q_out), _ptr(k_cache), _ptr(v_cache), n, nq, nkv, hd, rot_half,
-              int(page_size), dtype_code(x.dtype), _stream()), "rope_kv_write")
+              int(page_size), dtype_code(x.dtype), dtype_code(odt), _stream()), "rope_kv_write")
     return q_out
 
 

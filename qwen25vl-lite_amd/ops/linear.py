@@ -31,9 +31,10 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     out = skinny.try_linear(x, weight, bias, out_dtype)
     if out is not None:
         return out
-    y = torch.nn.functional.linear(x, weight)
     if out_dtype == torch.float32:
-        y = y.float()
+        y = torch.mm(x, weight.t(), out_dtype=torch.float32)  # float32 accumulator written out unrounded
+    else:
+        y = torch.nn.functional.linear(x, weight)
     if bias is not None:
         y = y + bias.to(y.dtype)
     return y

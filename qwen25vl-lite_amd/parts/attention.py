@@ -90,14 +90,16 @@ class PagedAttention(Mixer):
         if slot.writes == self.kv_shared:
             raise RuntimeError("a layer without key/value projections must read another layer's cache, "
                                "and a layer with them must write its own")
-        qkv = linear(x, self.w_in)
+        # Projections are written out in float32 (the accumulator, unrounded): bias, rotation and
+        # the residual sum then happen in float32 and each stored value is rounded once.
+        qkv = linear(x, self.w_in, out_dtype=torch.float32)
         inv_freq, freq_row = self.position.rotary_tables(self.hd)
         q = kernels.rope_kv_write(
             qkv, self.b_in, step.positions, inv_freq, freq_row,
             group.slot_mapping if write else None, slot.k_cache if write else None, slot.v_cache if write else None,
-            self.nq, self.nkv if write else 0, self.hd, group.page_size)
+            self.nq, self.nkv if write else 0, self.hd, group.page_size, out_dtype=self.dtype)
         o = paged_attention(q, slot.k_cache, slot.v_cache, group.block_table, step, self.nq, self.window, self.scale)
-        return linear(o, self.w_out)
+        return linear(o, self.w_out, out_dtype=torch.float32)
 
 
 register_part("mixer", "paged_attention", PagedAttention)

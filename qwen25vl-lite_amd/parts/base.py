@@ -120,7 +120,7 @@ class ResidualStream:
     norm adds ``pending`` to ``h`` in float32 in the same kernel that normalises."""
 
     h: torch.Tensor                          # float32 [N, hidden]
-    pending: Optional[torch.Tensor] = None   # run dtype [N, hidden]
+    pending: Optional[torch.Tensor] = None   # float32 or run dtype [N, hidden]
 
 
 class Part:

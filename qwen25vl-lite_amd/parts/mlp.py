@@ -44,7 +44,7 @@ class SwiGLU(FeedForward):
 
     def forward(self, x: torch.Tensor, step: StepContext) -> torch.Tensor:
         gate_up = linear(x, self.w_gate_up)
-        return linear(kernels.swiglu(gate_up), self.w_down)
+        return linear(kernels.swiglu(gate_up), self.w_down, out_dtype=torch.float32)
 
 
 register_part("ffn", "swiglu", SwiGLU)

@@ -1,0 +1,77 @@
+"""The device sampler: one token per logits row, chosen by a HIP kernel.
+
+The reference samples on the host, one request at a time (reference
+src/qwen25vl_lite/sampling.py:67-121, engine.py:802-829).  Here a step's rows are sampled
+together on the GPU; the only host work is the uniform random number of each row, which comes
+from the reference's per-token generator rule (seed + number of tokens generated so far).
+"""
+
+from __future__ import annotations
+
+import ctypes
+from typing import List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..ops.kernels import KernelError, _check, _fn, _stream
+from .params import SamplingParams
+
+__all__ = ["sample_rows", "uniform_for"]
+
+_ROW = np.dtype([("temperature", "<f4"), ("top_p", "<f4"), ("min_p", "<f4"), ("u", "<f4"),
+                 ("repetition", "<f4"), ("presence", "<f4"), ("frequency", "<f4"), ("top_k", "<i4"),
+                 ("prev_begin", "<i4"), ("prev_end", "<i4")])
+
+
+def uniform_for(params: SamplingParams, step: int) -> float:
+    """The uniform number in [0, 1) for a request's output token number ``step``."""
+    if params.temperature <= 0:
+        return 0.0
+    if params.seed is None:
+        return float(torch.rand(1).item())
+    gen = torch.Generator()
+    gen.manual_seed(int(params.seed) + int(step))
+    return float(torch.rand(1, generator=gen).item())
+
+
+def sample_rows(logits: torch.Tensor, params: Sequence[SamplingParams], prev_ids: Sequence[Sequence[int]],
+                steps: Sequence[int], uniforms: Optional[Sequence[float]] = None) -> List[int]:
+    """Sample a token for each row of float32 ``logits [M, vocab]`` on the GPU.
+
+    ``prev_ids[m]`` are the tokens request ``m`` has generated so far (for the penalties) and
+    ``steps[m]`` their number (for the seed rule).  ``uniforms`` overrides the random numbers.
+    """
+    if not logits.is_cuda:
+        raise KernelError("sampling has no CPU path: logits must be on the GPU")
+    if logits.dtype != torch.float32 or logits.dim() != 2 or not logits.is_contiguous():
+        raise KernelError("logits must be contiguous float32 [M, vocab]")
+    m, vocab = logits.shape
+    if not (len(params) == len(prev_ids) == len(steps) == m):
+        raise ValueError("one SamplingParams, token list and step per logits row is needed")
+    if m == 0:
+        return []
+    rows = np.zeros(m, _ROW)
+    flat: List[int] = []
+    for i, p in enumerate(params):
+        need_prev = p.repetition_penalty != 1.0 or p.presence_penalty != 0.0 or p.frequency_penalty != 0.0
+        begin = len(flat)
+        if need_prev:
+            flat.extend(int(t) for t in prev_ids[i])
+        u = uniforms[i] if uniforms is not None else uniform_for(p, steps[i])
+        rows[i] = (p.temperature, p.top_p, p.min_p, u, p.repetition_penalty, p.presence_penalty,
+                   p.frequency_penalty, p.top_k if p.top_k else -1, begin, len(flat))
+    fn = _fn("sample", "qvl_sample_rows",
+             [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
+              ctypes.c_int, ctypes.c_void_p])
+    dev = logits.device
+    with torch.cuda.device(dev):
+        packed = np.concatenate([rows.view(np.int32), np.asarray(flat or [0], np.int32)])
+        buf = torch.from_numpy(packed).to(dev)
+        n_row_words = rows.view(np.int32).size
+        need_scores = any(p.temperature > 0 or len(flat) for p in params)
+        scores = torch.empty_like(logits) if need_scores else logits
+        out = torch.empty(m, dtype=torch.int32, device=dev)
+        _check(fn(logits.data_ptr(), scores.data_ptr(), buf.data_ptr(), buf[n_row_words:].data_ptr(),
+                  out.data_ptr(), m, vocab, _stream()), "sample_rows")
+        return out.cpu().tolist()

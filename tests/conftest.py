@@ -71,9 +71,24 @@ def model_dirs(tmp_path_factory):
     in bfloat16 so that the float32 and the bfloat16 runs read the same values."""
     from qwen25vl_lite_amd import Qwen25VLConfig, write_random_model
 
+    from qwen25vl_lite_amd.weights import SafetensorsFile, write_safetensors
+
     out = {}
     for name, (raw, seed) in TINY.items():
         d = str(tmp_path_factory.mktemp(f"tiny_{name}"))
         write_random_model(Qwen25VLConfig.from_dict(raw), d, seed, dtype=torch.bfloat16)
         out[name] = d
+        # The same model with query and key projections scaled up: N(0, 0.02) weights give nearly
+        # uniform attention, which would hide a wrong key, window edge or page; these make the
+        # softmax peaked so that such faults show in the logits.
+        sharp = str(tmp_path_factory.mktemp(f"tiny_{name}_sharp"))
+        with SafetensorsFile(os.path.join(d, "model.safetensors")) as f:
+            tensors = {k: f.tensor(k).clone() for k in f.keys()}
+        for k in tensors:
+            if ".q_proj." in k or ".k_proj." in k:
+                tensors[k] = (tensors[k].float() * 7.0).to(torch.bfloat16)
+        write_safetensors(os.path.join(sharp, "model.safetensors"), tensors)
+        with open(os.path.join(d, "config.json")) as src, open(os.path.join(sharp, "config.json"), "w") as dst:
+            dst.write(src.read())
+        out[name + "_sharp"] = sharp
     return out

@@ -74,6 +74,15 @@ def plain_read_weights(model_dir: str) -> Dict[str, torch.Tensor]:
 # --------------------------------------------------------------------------------------------
 # the parts
 # --------------------------------------------------------------------------------------------
+def _keep(x: torch.Tensor) -> torch.Tensor:
+    return x
+
+
+def as_bfloat16(x: torch.Tensor) -> torch.Tensor:
+    """Round to bfloat16 and back: what storing a float32 value in bfloat16 does to it."""
+    return x.to(torch.bfloat16).to(torch.float32)
+
+
 def plain_rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     """reference layers.py:27-31: x * rsqrt(mean(x^2) + eps), then times the weight."""
     xf = x.float()
@@ -132,15 +141,17 @@ def plain_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: fl
     return torch.matmul(torch.softmax(scores, dim=-1), vv.float())
 
 
-def plain_mlp(x: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, down: torch.Tensor) -> torch.Tensor:
+def plain_mlp(x: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, down: torch.Tensor, store=_keep) -> torch.Tensor:
     """reference text.py:65-66: down(silu(gate(x)) * up(x)), no biases."""
-    return torch.nn.functional.linear(torch.nn.functional.silu(torch.nn.functional.linear(x, gate))
-                                      * torch.nn.functional.linear(x, up), down)
+    lin = torch.nn.functional.linear
+    return lin(store(torch.nn.functional.silu(store(lin(x, gate))) * store(lin(x, up))), down)
 
 
 def plain_attention_layer(x: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str, cfg: dict,
-                          position_ids: torch.Tensor, window: Optional[int]) -> torch.Tensor:
-    """reference text.py:85-90 (projections, heads), :118 (rotation), :78 (scale), :177-178."""
+                          position_ids: torch.Tensor, window: Optional[int], store=_keep) -> torch.Tensor:
+    """reference text.py:85-90 (projections, heads), :118 (rotation), :78 (scale), :177-178.
+    ``store`` is applied where a bfloat16 run stores a value: rotated queries and keys, values,
+    the attention output (reference text.py:125-126 writes k and v to the cache in its dtype)."""
     t = x.shape[0]
     nh, nkv, hd = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
     lin = torch.nn.functional.linear
@@ -149,14 +160,20 @@ def plain_attention_layer(x: torch.Tensor, w: Dict[str, torch.Tensor], prefix: s
     v = lin(x, w[prefix + "v_proj.weight"], w[prefix + "v_proj.bias"]).view(t, nkv, hd).transpose(0, 1)
     cos, sin = plain_mrope_cos_sin(position_ids, plain_inv_freq(hd, cfg["rope_theta"]))
     q, k = plain_apply_mrope(q, k, cos, sin, cfg["mrope_section"])
-    o = plain_attention(q, k, v, hd ** -0.5, window)
+    o = store(plain_attention(store(q), store(k), store(v), hd ** -0.5, window))
     return lin(o.transpose(0, 1).reshape(t, nh * hd), w[prefix + "o_proj.weight"])
 
 
 def plain_forward(cfg: dict, w: Dict[str, torch.Tensor], token_ids: Sequence[int],
-                  position_ids: Optional[torch.Tensor] = None) -> torch.Tensor:
+                  position_ids: Optional[torch.Tensor] = None, store=_keep) -> torch.Tensor:
     """Logits [T, vocab] of a whole sequence (reference text.py:196-206, 264-279; model.py:84-86,
-    200-202).  Text positions: 0..T-1 on all three rows (reference rope.py:194-197)."""
+    200-202).  Text positions: 0..T-1 on all three rows (reference rope.py:194-197).
+
+    ``store`` models a run whose activations are stored in a narrower type: it is applied to the
+    normalised activations, to q, k, v and the attention output, and to the feed-forward's
+    inner values, i.e. to every operand of a matrix product and to what the cache holds (the
+    reference runs all of these in its model dtype).  The residual sum, the norms' statistics
+    and the logits stay float32.  ``as_bfloat16`` gives what a bfloat16 run can be held to."""
     ids = torch.tensor(list(token_ids), dtype=torch.long)
     t = ids.shape[0]
     if position_ids is None:
@@ -167,19 +184,20 @@ def plain_forward(cfg: dict, w: Dict[str, torch.Tensor], token_ids: Sequence[int
     h = w["embed_tokens.weight"][ids]
     for i in range(cfg["num_hidden_layers"]):
         p = f"layers.{i}."
-        a = plain_attention_layer(plain_rmsnorm(h, w[p + "input_layernorm.weight"], eps), w, p + "self_attn.",
-                                  cfg, position_ids, windows[i])
+        a = plain_attention_layer(store(plain_rmsnorm(h, w[p + "input_layernorm.weight"], eps)), w,
+                                  p + "self_attn.", cfg, position_ids, windows[i], store)
         h = h + a
-        m = plain_mlp(plain_rmsnorm(h, w[p + "post_attention_layernorm.weight"], eps),
-                      w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+        m = plain_mlp(store(plain_rmsnorm(h, w[p + "post_attention_layernorm.weight"], eps)),
+                      w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"],
+                      store)
         h = h + m
-    h = plain_rmsnorm(h, w["norm.weight"], eps)
+    h = store(plain_rmsnorm(h, w["norm.weight"], eps))
     head = w["lm_head.weight"] if "lm_head.weight" in w else w["embed_tokens.weight"]
     return torch.nn.functional.linear(h, head)
 
 
-def plain_model_logits(model_dir: str, token_ids: Sequence[int], position_ids=None) -> torch.Tensor:
-    return plain_forward(plain_read_config(model_dir), plain_read_weights(model_dir), token_ids, position_ids)
+def plain_model_logits(model_dir: str, token_ids: Sequence[int], position_ids=None, store=_keep) -> torch.Tensor:
+    return plain_forward(plain_read_config(model_dir), plain_read_weights(model_dir), token_ids, position_ids, store)
 
 
 # --------------------------------------------------------------------------------------------

@@ -1,0 +1,171 @@
+"""Generation through the entry points, the sampler kernel, and the trace_run program."""
+
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+from plain_model import plain_filtered_probs, plain_model_logits, plain_penalties
+from replay_util import random_tokens
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _plain_greedy(model_dir, prompt, n):
+    ids, out = list(prompt), []
+    for _ in range(n):
+        nxt = int(torch.argmax(plain_model_logits(model_dir, ids)[-1]))
+        out.append(nxt)
+        ids.append(nxt)
+    return out
+
+
+@pytest.mark.parametrize("name, dtype", [("A", "float32"), ("B_sharp", "float32"), ("C_sharp", "float32")])
+def test_greedy_generation_through_llm(model_dirs, name, dtype):
+    # reference tests/test_engine.py:36-54 (prompt 3..12, 8 tokens), and batched = alone (test_chunked_prefill.py:155-190)
+    from qwen25vl_lite_amd import LLM, SamplingParams
+
+    d = model_dirs[name]
+    vocab = {"A": 256, "B": 509, "C": 300}[name[0]]
+    prompts = [list(range(3, 13)), random_tokens(6, vocab, 1), random_tokens(3, vocab, 2), random_tokens(45, vocab, 3)]
+    llm = LLM(d, dtype=dtype, num_blocks=32, block_size=16, max_num_seqs=3, max_num_batched_tokens=24)
+    outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True))
+    for prompt, out in zip(prompts, outs):
+        assert out.prompt_token_ids == prompt and out.finish_reason == "length"
+        assert out.output_token_ids == _plain_greedy(d, prompt, 8)
+    assert llm.runner.cache.pages_in_use()[0] == (len(llm.runner.cache.prefix_cache)
+                                                  if llm.runner.cache.prefix_cache else 0)
+    llm.runner.cache.check()
+
+
+def test_long_decode_and_preemption(model_dirs):
+    """Decoding well past several pages, with so few pages that requests are preempted and
+    prefilled again: the tokens are still the plain implementation's."""
+    from qwen25vl_lite_amd import LLM, SamplingParams
+
+    d = model_dirs["B_sharp"]
+    prompts = [random_tokens(20, 509, 10 + i) for i in range(3)]
+    llm = LLM(d, dtype="float32", num_blocks=10, block_size=16, max_num_seqs=3, max_num_batched_tokens=32,
+              enable_prefix_cache=False)
+    outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=70, ignore_eos=True))
+    assert llm.engine.stats()["preemptions"] > 0
+    for prompt, out in zip(prompts, outs):
+        assert out.output_token_ids == _plain_greedy(d, prompt, 70)
+    assert llm.runner.cache.pages_in_use() == [0, 0]
+
+
+def test_prefix_reuse_gives_the_same_tokens(model_dirs):
+    # reference tests/test_chunked_prefill.py:193-227, tests/test_engine.py:57-106
+    from qwen25vl_lite_amd import LLM, SamplingParams
+
+    d = model_dirs["A_sharp"]
+    shared = random_tokens(40, 256, 77)
+    llm = LLM(d, dtype="float32", num_blocks=32, block_size=16, max_num_seqs=2)
+    params = SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True)
+    first = llm.generate([shared + [1, 2, 3]], params)[0]
+    second = llm.generate([shared + [9, 8]], params)[0]
+    assert second.metrics["cached_tokens"] == 32 and first.metrics["cached_tokens"] == 0
+    assert second.output_token_ids == _plain_greedy(d, shared + [9, 8], 6)
+    assert first.output_token_ids == _plain_greedy(d, shared + [1, 2, 3], 6)
+
+
+def test_temperature_sampling_is_seeded_and_batch_independent(model_dirs):
+    from qwen25vl_lite_amd import LLM, SamplingParams
+
+    d = model_dirs["B"]
+    prompts = [random_tokens(n, 509, 30 + n) for n in (1, 9, 40)]
+    params = SamplingParams(temperature=0.7, max_tokens=12, seed=1, ignore_eos=True)
+    llm = LLM(d, dtype="float32", num_blocks=32, block_size=16, max_num_seqs=4, max_num_batched_tokens=7)
+    together = [o.output_token_ids for o in llm.generate(prompts, params)]
+    alone = [llm.generate([p], params)[0].output_token_ids for p in prompts]
+    assert together == alone
+    other = llm.generate([prompts[2]], SamplingParams(temperature=0.7, max_tokens=12, seed=2, ignore_eos=True))[0]
+    assert other.output_token_ids != together[2]
+
+
+def _plain_draw(logits, prev, p, u):
+    pen = plain_penalties(logits, prev, p.repetition_penalty, p.presence_penalty, p.frequency_penalty)
+    if p.temperature <= 0:
+        return int(torch.argmax(pen))
+    probs = plain_filtered_probs(pen, p.temperature, p.top_k, p.top_p, p.min_p)
+    cdf = torch.cumsum(probs.double(), 0)
+    return int(torch.searchsorted(cdf, torch.tensor(u * float(cdf[-1]), dtype=torch.float64), right=True).clamp(max=len(probs) - 1))
+
+
+def test_sampler_kernel_against_plain():
+    from qwen25vl_lite_amd.sampling import SamplingParams
+    from qwen25vl_lite_amd.sampling.sampler import sample_rows
+
+    g = torch.Generator().manual_seed(0)
+    vocab = 1531
+    cases = [
+        SamplingParams(temperature=0.0),
+        SamplingParams(temperature=0.0, repetition_penalty=1.7, presence_penalty=0.4, frequency_penalty=0.3),
+        SamplingParams(temperature=1.0),
+        SamplingParams(temperature=0.7, top_k=5),
+        SamplingParams(temperature=1.3, top_p=0.6),
+        SamplingParams(temperature=0.9, min_p=0.1),
+        SamplingParams(temperature=0.8, top_k=40, top_p=0.9, min_p=0.02, repetition_penalty=1.2),
+        SamplingParams(temperature=1.0, top_k=1),
+    ]
+    for trial in range(6):
+        logits = torch.randn(len(cases), vocab, generator=g) * 3
+        prev = [torch.randint(0, vocab, (trial * 7,), generator=g).tolist() for _ in cases]
+        us = torch.rand(len(cases), generator=g).tolist()
+        got = sample_rows(logits.cuda(), cases, prev, [len(p) for p in prev], uniforms=us)
+        for i, p in enumerate(cases):
+            want = _plain_draw(logits[i], prev[i], p, us[i])
+            if got[i] != want:
+                # a draw that lands within rounding of a boundary of the distribution function
+                probs = plain_filtered_probs(plain_penalties(logits[i], prev[i], p.repetition_penalty,
+                                                             p.presence_penalty, p.frequency_penalty),
+                                             max(p.temperature, 1e-6), p.top_k, p.top_p, p.min_p).double()
+                cdf = torch.cumsum(probs, 0) / probs.sum()
+                assert probs[got[i]] > 0 and min(abs(cdf[got[i]] - us[i]), abs(cdf[got[i]] - probs[got[i]] - us[i])) < 1e-5, \
+                    (trial, i, got[i], want)
+    # the distribution itself: many draws of one row follow the filtered probabilities
+    p = SamplingParams(temperature=1.0, top_k=4)
+    row = torch.tensor([2.0, 1.0, 0.5, 0.0, -1.0, -3.0])
+    n = 4000
+    us = ((torch.arange(n) + 0.5) / n).tolist()
+    draws = sample_rows(row.repeat(n, 1).cuda(), [p] * n, [[]] * n, [0] * n, uniforms=us)
+    freq = torch.bincount(torch.tensor(draws), minlength=6).double() / n
+    assert torch.allclose(freq, plain_filtered_probs(row, 1.0, top_k=4).double(), atol=2e-3)
+
+
+def test_trace_run_program(model_dirs, tmp_path):
+    """bin/trace_run as a user calls it: JSON steps on standard input, `done <step>` lines,
+    <step>.f32 files of little-endian float32 [wanted, vocab]."""
+    d = model_dirs["A"]
+    toks = random_tokens(21, 256, 4)
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": toks[:9], "want": [0, 8]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": toks[9:20], "want": []}], "end": []},
+        {"step": 2, "entries": [{"id": "a", "tokens": toks[20:], "want": [0]},
+                                {"id": "b", "tokens": toks[:3], "want": [2]}], "end": ["a", "b"]},
+    ]
+    out = tmp_path / "out"
+    proc = subprocess.run(
+        [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", d, "--dtype", "float32", "--out", str(out),
+         "--max-tokens", "128"],
+        input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=110)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert proc.stdout.split() == ["done", "0", "done", "1", "done", "2"]
+    assert sorted(os.listdir(out)) == ["0.f32", "2.f32"]
+    ref = plain_model_logits(d, toks)
+    import numpy as np
+    s0 = torch.from_numpy(np.fromfile(out / "0.f32", dtype="<f4").reshape(2, 256))
+    s2 = torch.from_numpy(np.fromfile(out / "2.f32", dtype="<f4").reshape(2, 256))
+    assert torch.allclose(s0, ref[[0, 8]], atol=1e-4, rtol=1e-3)
+    assert torch.allclose(s2[0], ref[20], atol=1e-4, rtol=1e-3) and torch.allclose(s2[1], ref[2], atol=1e-4, rtol=1e-3)
+
+
+def test_smoke_entry():
+    sys.path.insert(0, ROOT)
+    import __graft_entry__
+    __graft_entry__.smoke()

@@ -1,0 +1,208 @@
+"""Each HIP kernel alone against a plain float32 formula, at sizes other than the engine's."""
+
+import math
+
+import pytest
+import torch
+
+from plain_model import (plain_apply_mrope, plain_attention, plain_inv_freq, plain_mrope_cos_sin, plain_rmsnorm)
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def _tol(dtype):
+    return dict(atol=1e-5, rtol=1e-5) if dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embed_gather(dtype):
+    from qwen25vl_lite_amd.ops import kernels
+    torch.manual_seed(0)
+    table = torch.randn(301, 100).to(dtype).cuda()
+    ids = torch.tensor([0, 300, 7, 7, 150], dtype=torch.int32).cuda()
+    out = kernels.embed_gather(ids, table)
+    assert out.dtype == torch.float32 and torch.equal(out, table[ids.long()].float())
+
+
+@pytest.mark.parametrize("width", [97, 3584, 8200])
+@pytest.mark.parametrize("delta_dtype, out_dtype", [(torch.float32, torch.float32), (torch.float32, torch.bfloat16),
+                                                    (torch.bfloat16, torch.bfloat16), (None, torch.bfloat16)])
+def test_add_rmsnorm(width, delta_dtype, out_dtype):
+    from qwen25vl_lite_amd.ops import kernels
+    torch.manual_seed(width)
+    n, eps = 5, 1e-5
+    h = torch.randn(n, width) * 3
+    delta = torch.randn(n, width).to(delta_dtype) if delta_dtype is not None else None
+    w = 1 + 0.1 * torch.randn(width)
+    total = h + (delta.float() if delta is not None else 0)
+    want = plain_rmsnorm(total, w, eps)
+    hd = h.cuda()
+    out = kernels.add_rmsnorm(hd, None if delta is None else delta.cuda(), w.cuda(), eps, out_dtype)
+    assert out.dtype == out_dtype
+    assert torch.allclose(out.float().cpu(), want, **_tol(out_dtype))
+    assert torch.allclose(hd.cpu(), total, atol=1e-6), "the sum is written back in float32"
+    # selected rows: h stays as it was
+    hd = h.cuda()
+    rows = torch.tensor([4, 0, 4], dtype=torch.int32).cuda()
+    out = kernels.add_rmsnorm(hd, None if delta is None else delta.cuda(), w.cuda(), eps, out_dtype, rows=rows)
+    assert torch.allclose(out.float().cpu(), want[[4, 0, 4]], **_tol(out_dtype)) and torch.equal(hd.cpu(), h)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq, nkv, hd, sections", [(6, 2, 24, (4, 4, 4)), (5, 1, 48, (10, 6, 8)), (4, 4, 128, (16, 24, 24))])
+def test_rope_kv_write(dtype, nq, nkv, hd, sections):
+    from qwen25vl_lite_amd.ops import kernels
+    torch.manual_seed(hd)
+    n, ps, pages, theta = 11, 16, 5, 1e4
+    x = torch.randn(n, (nq + 2 * nkv) * hd)
+    bias = torch.randn((nq + 2 * nkv) * hd) * 0.1
+    pos = torch.stack([torch.randint(0, 5000, (n,)) for _ in range(3)])
+    slots = torch.randperm(pages * ps)[:n].to(torch.int32)
+    inv = plain_inv_freq(hd, theta)
+    rows = torch.tensor(sum(([r] * c for r, c in enumerate(sections)), []), dtype=torch.int32)
+    kc = torch.zeros(pages, nkv, ps, hd, dtype=dtype).cuda()
+    vc = torch.zeros(pages, nkv, hd, ps, dtype=dtype).cuda()
+    q = kernels.rope_kv_write(x.cuda(), bias.cuda(), pos.to(torch.int32).cuda(), inv.cuda(), rows.cuda(), slots.cuda(),
+                              kc, vc, nq, nkv, hd, ps, out_dtype=dtype)
+    xb = x + bias
+    qs, ks, vs = xb.split([nq * hd, nkv * hd, nkv * hd], dim=1)
+    cos, sin = plain_mrope_cos_sin(pos, inv)
+    qr, kr = plain_apply_mrope(qs.view(n, nq, hd).transpose(0, 1), ks.view(n, nkv, hd).transpose(0, 1), cos, sin, sections)
+    tol = dict(atol=2e-4, rtol=1e-4) if dtype == torch.float32 else _tol(dtype)   # sin/cos of angles up to 5000
+    assert torch.allclose(q.float().cpu().view(n, nq, hd), qr.transpose(0, 1), **tol)
+    kflat = kc.float().cpu().permute(0, 2, 1, 3).reshape(pages * ps, nkv, hd)          # [slot, kv head, hd]
+    vflat = vc.float().cpu().permute(0, 3, 1, 2).reshape(pages * ps, nkv, hd)
+    assert torch.allclose(kflat[slots.long()], kr.transpose(0, 1), **tol)
+    assert torch.allclose(vflat[slots.long()], vs.view(n, nkv, hd), **_tol(dtype))
+    untouched = torch.ones(pages * ps, dtype=torch.bool)
+    untouched[slots.long()] = False
+    assert kflat[untouched].abs().max() == 0 and vflat[untouched].abs().max() == 0
+    # position 0 leaves a head as it is; a negative slot writes nothing; rot < hd leaves the tail alone
+    kc.zero_()
+    q0 = kernels.rope_kv_write(x.cuda(), None, torch.zeros(3, n, dtype=torch.int32).cuda(), inv.cuda(), rows.cuda(),
+                               torch.full((n,), -1, dtype=torch.int32).cuda(), kc, vc, nq, nkv, hd, ps, out_dtype=dtype)
+    assert torch.allclose(q0.float().cpu(), x[:, :nq * hd].to(dtype).float(), atol=1e-6) and kc.abs().max() == 0
+    half = hd // 4
+    qp = kernels.rope_kv_write(x[:, :nq * hd].contiguous().cuda(), None, pos.to(torch.int32).cuda(),
+                               plain_inv_freq(2 * half, theta).cuda(), torch.zeros(half, dtype=torch.int32).cuda(),
+                               None, None, None, nq, 0, hd, ps, out_dtype=dtype)
+    qp = qp.float().cpu().view(n, nq, hd)
+    assert torch.allclose(qp[..., 2 * half:], x[:, :nq * hd].view(n, nq, hd)[..., 2 * half:].to(dtype).float(), atol=1e-6)
+    c1, s1 = plain_mrope_cos_sin(pos[:1].expand(3, n), plain_inv_freq(2 * half, theta))
+    want, _ = plain_apply_mrope(x[:, :nq * hd].view(n, nq, hd)[..., :2 * half].transpose(0, 1),
+                                x[:, :nq * hd].view(n, nq, hd)[..., :2 * half].transpose(0, 1), c1, s1, (half, 0, 0))
+    assert torch.allclose(qp[..., :2 * half], want.transpose(0, 1), **tol)
+
+
+def _paged(k, v, ps, pages, dtype, seed):
+    """Scatter per-request keys/values [nkv, T, hd] into shuffled pages; returns caches and tables."""
+    g = torch.Generator().manual_seed(seed)
+    nkv, hd = k[0].shape[0], k[0].shape[2]
+    kc = torch.randn(pages, nkv, ps, hd, generator=g).to(dtype)          # stale values everywhere
+    vc = torch.randn(pages, nkv, hd, ps, generator=g).to(dtype)
+    order = torch.randperm(pages, generator=g).tolist()
+    width = max((x.shape[1] + ps - 1) // ps for x in k)
+    table = torch.full((len(k), width), -1, dtype=torch.int32)
+    for r, (kr, vr) in enumerate(zip(k, v)):
+        for i in range((kr.shape[1] + ps - 1) // ps):
+            page = order.pop()
+            table[r, i] = page
+            n = min(ps, kr.shape[1] - i * ps)
+            kc[page, :, :n] = kr[:, i * ps:i * ps + n].to(dtype)
+            vc[page, :, :, :n] = vr[:, i * ps:i * ps + n].transpose(1, 2).to(dtype)
+    return kc, vc, table
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq, nkv, hd, window", [(6, 2, 24, None), (5, 1, 48, 40), (8, 8, 16, 7), (14, 2, 128, None),
+                                                 (4, 2, 80, 130)])
+def test_paged_attention_generic(dtype, nq, nkv, hd, window):
+    """Prompt portions and single tokens of several requests in one call, pages shuffled, stale
+    values in every unused slot.  One query and one far key are scaled so that a single score
+    dominates: a kernel that misses that key (a page, a window edge) fails by far."""
+    from qwen25vl_lite_amd.ops import kernels
+    torch.manual_seed(nq * hd)
+    ps = 16
+    lens = [333, 17, 64, 1]           # context of each request after this step
+    qlens = [5, 17, 1, 1]             # of which the last qlen are this step's tokens
+    k = [torch.randn(nkv, t, hd) for t in lens]
+    v = [torch.randn(nkv, t, hd) for t in lens]
+    k = [x.to(dtype).float() for x in k]
+    v = [x.to(dtype).float() for x in v]
+    q_all = [torch.randn(nq, t, hd) for t in lens]
+    far = 2 if window is None else max(0, 332 - window + 1)      # the first key the last query still sees
+    kf = k[0][:, far].repeat_interleave(nq // nkv, 0)
+    q_all[0][:, 332] = kf * (30.0 / (kf.pow(2).sum(-1, keepdim=True) * hd ** -0.5))      # that score is 30
+    q_all = [x.to(dtype).float() for x in q_all]
+    scale = hd ** -0.5
+    kc, vc, table = _paged(k, v, ps, 40, dtype, 1)
+    qs, req, seqpos, want = [], [], [], []
+    for r, (t, ql) in enumerate(zip(lens, qlens)):
+        full = plain_attention(q_all[r], k[r], v[r], scale, window)      # [nq, t, hd]
+        for p in range(t - ql, t):
+            qs.append(q_all[r][:, p].reshape(-1))
+            req.append(r)
+            seqpos.append(p)
+            want.append(full[:, p].reshape(-1))
+    q = torch.stack(qs).to(dtype).cuda()
+    out = kernels.paged_attention_generic(q, kc.cuda(), vc.cuda(), table.cuda(),
+                                          torch.tensor(req, dtype=torch.int32).cuda(),
+                                          torch.tensor(seqpos, dtype=torch.int32).cuda(), nq, window, scale)
+    want = torch.stack(want)
+    tol = dict(atol=2e-5, rtol=1e-4) if dtype == torch.float32 else dict(atol=1.5e-2, rtol=2e-2)
+    assert torch.allclose(out.float().cpu(), want, **tol), (out.float().cpu() - want).abs().max()
+    # the dominated row really is dominated by the far key's value
+    row = 4  # request 0, position 332
+    assert torch.allclose(want[row].view(nq, hd), v[0][:, far].repeat_interleave(nq // nkv, 0), atol=1e-3)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_swiglu(dtype):
+    from qwen25vl_lite_amd.ops import kernels
+    torch.manual_seed(3)
+    x = (torch.randn(7, 2 * 353) * 3).to(dtype)
+    want = torch.nn.functional.silu(x[:, :353].float()) * x[:, 353:].float()
+    out = kernels.swiglu(x.cuda())
+    assert torch.allclose(out.float().cpu(), want, **_tol(dtype))
+
+
+@pytest.mark.parametrize("m, n, k", [(1, 5, 3), (7, 509, 144), (65, 130, 353), (130, 64, 1000)])
+def test_gemm_f32_is_exact_and_row_independent(m, n, k):
+    from qwen25vl_lite_amd.ops import kernels
+    torch.manual_seed(m)
+    x, w, b = torch.randn(m, k), torch.randn(n, k), torch.randn(n)
+    want = (x.double() @ w.double().T + b.double()).float()
+    out = kernels.gemm_f32(x.cuda(), w.cuda(), b.cuda())
+    assert torch.allclose(out.cpu(), want, atol=1e-4 * math.sqrt(k), rtol=1e-5)
+    # no reduced-precision input format: products of values that bfloat16/tf32 would round
+    xe = torch.full((1, 4), 1 + 2 ** -20)
+    we = torch.tensor([[1.0, -1.0, 1.0, -1.0 + 2 ** -19]])
+    assert kernels.gemm_f32(xe.cuda(), we.cuda()).item() == pytest.approx((xe.double() @ we.double().T).item(), abs=1e-12)
+    # a row's result does not depend on what else is in the batch
+    alone = kernels.gemm_f32(x[m // 2:m // 2 + 1].contiguous().cuda(), w.cuda(), b.cuda())
+    assert torch.equal(alone[0], out[m // 2])
+
+
+@pytest.mark.parametrize("m, n, k", [(1, 509, 144), (8, 300, 200), (33, 130, 352), (300, 64, 1000)])
+def test_linear_bfloat16(m, n, k):
+    from qwen25vl_lite_amd.ops.linear import linear
+    torch.manual_seed(k)
+    x, w = torch.randn(m, k).bfloat16(), (torch.randn(n, k) / math.sqrt(k)).bfloat16()
+    want = x.float() @ w.float().T
+    out32 = linear(x.cuda(), w.cuda(), out_dtype=torch.float32)
+    assert out32.dtype == torch.float32 and torch.allclose(out32.cpu(), want, atol=2e-3, rtol=2e-3)
+    out16 = linear(x.cuda(), w.cuda())
+    assert out16.dtype == torch.bfloat16 and torch.allclose(out16.float().cpu(), want, atol=2e-2, rtol=2e-2)
+
+
+def test_no_cpu_path():
+    from qwen25vl_lite_amd.ops import kernels
+    from qwen25vl_lite_amd.ops.linear import linear
+    with pytest.raises(kernels.KernelError):
+        kernels.swiglu(torch.zeros(2, 4))
+    with pytest.raises(kernels.KernelError):
+        linear(torch.zeros(2, 4), torch.zeros(3, 4))
+    with pytest.raises(kernels.KernelError):
+        kernels.swiglu(torch.zeros(2, 4, dtype=torch.float16).cuda())

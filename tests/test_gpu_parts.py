@@ -1,0 +1,321 @@
+"""Each part alone, and parts defined here (a mixer with state of its own, a routed feed-forward,
+another position encoding) registered, built and stepped without touching the framework."""
+
+import math
+
+import pytest
+import torch
+
+from plain_model import plain_attention, plain_inv_freq, plain_rmsnorm
+
+pytestmark = pytest.mark.gpu
+
+
+def _spec_model(layers, hidden, vocab, dtype=torch.float32, run=None, seed=0):
+    from qwen25vl_lite_amd.models import DecoderModel, LayerSpec, ModelSpec, RunEntry
+    from qwen25vl_lite_amd.parts import PartSpec
+    from qwen25vl_lite_amd.weights import fill_random
+
+    norm = PartSpec("rms_norm", {"size": hidden, "eps": 1e-6})
+    specs = []
+    for i, (mixer, ffn) in enumerate(layers):
+        block = PartSpec("pre_norm", {"norm1": norm, "mixer": mixer, "norm2": norm, "ffn": ffn,
+                                      "names": {"norm1": "ln1", "mixer": "mix", "norm2": "ln2", "ffn": "ff"}})
+        specs.append(LayerSpec(block, f"blocks.{i}."))
+    spec = ModelSpec(hidden_size=hidden, vocab_size=vocab, layers=specs,
+                     run=run or [RunEntry(i) for i in range(len(layers))], final_norm=norm,
+                     tie_word_embeddings=True, position_rows=3, embed_name="tok.weight", final_norm_prefix="ln_f.")
+    model = DecoderModel(spec, dtype, "cuda:0")
+    fill_random(model, seed, std=0.3)
+    return model
+
+
+def _runner(model, pages=32, seqs=4):
+    from qwen25vl_lite_amd.config import EngineConfig
+    from qwen25vl_lite_amd.engine import ModelRunner
+    ecfg = EngineConfig(num_blocks=pages, block_size=16, max_num_seqs=seqs, max_num_batched_tokens=512,
+                        max_model_len=pages * 16, enable_prefix_cache=False, dtype=model.dtype)
+    return ModelRunner(model, ecfg)
+
+
+def _run(runner, rid, tokens, cuts):
+    from qwen25vl_lite_amd.engine import StepEntry
+    runner.admit(rid)
+    rows, at = [], 0
+    for c in cuts:
+        part = tokens[at:at + c]
+        rows.append(runner.execute([StepEntry(rid, part, at, want=list(range(len(part))))]).cpu())
+        at += len(part)
+    assert at == len(tokens)
+    runner.release(rid)
+    return torch.cat(rows)
+
+
+def _attn_spec(hidden, nq, nkv, hd, position, window=None, scale=None):
+    from qwen25vl_lite_amd.parts import PartSpec
+    return PartSpec("paged_attention", {"hidden_size": hidden, "num_heads": nq, "num_kv_heads": nkv, "head_dim": hd,
+                                        "qkv_bias": False, "window": window, "scale": scale, "position": position})
+
+
+def test_norm_part_alone():
+    from qwen25vl_lite_amd.parts import PartSpec, ResidualStream, build_part
+    torch.manual_seed(0)
+    part = build_part("norm", PartSpec("rms_norm", {"size": 70, "eps": 1e-3}), torch.float32, torch.device("cuda:0"))
+    assert {k: v.shape for k, v in part.param_specs().items()} == {"weight": (70,)}
+    w = torch.randn(70)
+    part.load({"weight": w.cuda()})
+    h, d = torch.randn(4, 70), torch.randn(4, 70)
+    stream = ResidualStream(h.cuda(), d.cuda())
+    out = part.forward(stream)
+    assert stream.pending is None and torch.allclose(stream.h.cpu(), h + d, atol=1e-6)
+    assert torch.allclose(out.cpu(), plain_rmsnorm(h + d, w, 1e-3), atol=1e-5)
+
+
+def test_position_parts_alone():
+    from qwen25vl_lite_amd.parts import PartSpec, build_part
+    dev = torch.device("cuda:0")
+    mrope = build_part("position", PartSpec("mrope", {"theta": 1e4, "sections": (2, 3, 3)}), torch.float32, dev)
+    inv, rows = mrope.rotary_tables(16)
+    assert rows.tolist() == [0, 0, 1, 1, 1, 2, 2, 2] and torch.equal(inv.cpu(), plain_inv_freq(16, 1e4))
+    with pytest.raises(ValueError):
+        mrope.rotary_tables(32)        # sections must cover half the head (reference rope.py:89-93)
+    rope = build_part("position", PartSpec("rope", {"theta": 1e4, "rotary_dim": 8}), torch.float32, dev)
+    inv, rows = rope.rotary_tables(16)
+    assert rows.tolist() == [0] * 4 and torch.equal(inv.cpu(), plain_inv_freq(8, 1e4))
+
+
+def test_feed_forward_part_alone():
+    from qwen25vl_lite_amd.parts import PartSpec, build_part
+    torch.manual_seed(1)
+    part = build_part("ffn", PartSpec("swiglu", {"hidden_size": 40, "intermediate_size": 72}), torch.float32,
+                      torch.device("cuda:0"))
+    g, u, d = torch.randn(72, 40), torch.randn(72, 40), torch.randn(40, 72)
+    part.load({"gate_proj.weight": g.cuda(), "up_proj.weight": u.cuda(), "down_proj.weight": d.cuda()})
+    x = torch.randn(5, 40)
+    want = (torch.nn.functional.silu(x @ g.T) * (x @ u.T)) @ d.T
+    assert torch.allclose(part.forward(x.cuda(), None).cpu(), want, atol=1e-4)
+    assert torch.equal(part.named_weights()["up_proj.weight"].cpu(), u)
+
+
+def test_attention_part_without_rotation_is_plain_attention():
+    """One layer whose position encoding rotates nothing (rotary_dim 0) and a custom scale: the
+    mixer reduces to causal attention over the projections, computed here with the library."""
+    from qwen25vl_lite_amd.parts import PartSpec
+    hidden, nq, nkv, hd = 48, 4, 2, 12
+    pos = PartSpec("rope", {"theta": 1e4, "rotary_dim": 0})
+    ffn = PartSpec("swiglu", {"hidden_size": hidden, "intermediate_size": 16})
+    model = _spec_model([(_attn_spec(hidden, nq, nkv, hd, pos, scale=0.37), ffn)], hidden, 50)
+    mixer = model.blocks[0].mixer
+    w = {k: v.float().cpu() for k, v in mixer.named_weights().items()}
+    torch.manual_seed(2)
+    t = 37
+    x = torch.randn(t, hidden)
+    from qwen25vl_lite_amd.engine import StepEntry
+    from qwen25vl_lite_amd.engine.batch import build_step
+    runner = _runner(model)
+    runner.admit("a")
+    runner.cache.reserve("a", t)
+    step = build_step([StepEntry("a", [0] * t, 0)], runner.cache, 3, torch.float32, model.device)
+    out = mixer.forward(x.cuda(), step, runner.slots[0]).cpu()
+    q = (x @ w["q_proj.weight"].T).view(t, nq, hd).transpose(0, 1)
+    k = (x @ w["k_proj.weight"].T).view(t, nkv, hd).transpose(0, 1)
+    v = (x @ w["v_proj.weight"].T).view(t, nkv, hd).transpose(0, 1)
+    lib = torch.nn.functional.scaled_dot_product_attention(
+        q[None], k.repeat_interleave(2, 0)[None], v.repeat_interleave(2, 0)[None], is_causal=True, scale=0.37)[0]
+    want = lib.transpose(0, 1).reshape(t, nq * hd) @ w["o_proj.weight"].T
+    assert torch.allclose(out, want, atol=1e-4)
+
+
+def test_a_layer_named_twice_and_a_layer_reading_anothers_cache():
+    """Run list [0, 1, 0, 2->cache of entry 1]: layer 0 runs twice with caches of its own, the last
+    entry has no key/value projections and attends over what entry 1 wrote.  Cutting the sequence
+    differently must not change a logit."""
+    from qwen25vl_lite_amd.models import RunEntry
+    from qwen25vl_lite_amd.parts import PartSpec
+    hidden = 32
+    pos = PartSpec("mrope", {"theta": 100.0, "sections": (1, 2, 1)})
+    ffn = PartSpec("swiglu", {"hidden_size": hidden, "intermediate_size": 40})
+    full = _attn_spec(hidden, 4, 2, 8, pos)
+    shared = PartSpec("paged_attention", dict(full.params, kv_shared=True))
+    model = _spec_model([(full, ffn), (full, ffn), (shared, ffn)], hidden, 60,
+                        run=[RunEntry(0), RunEntry(1), RunEntry(0), RunEntry(2, cache_from=1)])
+    assert model.cache_groups()[0].num_layers == 3 and "blocks.2.mix.k_proj.weight" not in model.expected_tensors()
+    runner = _runner(model)
+    toks = torch.randint(0, 60, (45,), generator=torch.Generator().manual_seed(3)).tolist()
+    whole = _run(runner, "w", toks, [45])
+    cut = _run(runner, "c", toks, [7, 2, 20, 1, 1, 14])
+    assert torch.allclose(whole, cut, atol=1e-5)
+    assert not torch.allclose(whole[1:], whole[:-1], atol=1e-3)
+
+
+# ---------------------------------------------------------------------------------------------
+# parts defined in the test
+# ---------------------------------------------------------------------------------------------
+def _register_toys():
+    from qwen25vl_lite_amd.parts import (FeedForward, Mixer, ParamSpec, PositionEncoding, StateNeed, known_parts,
+                                         register_part)
+    if "toy_decay" in known_parts("mixer"):
+        return
+
+    class DecayMixer(Mixer):
+        """y_t = s_t,  s_t = a * s_{t-1} + B x_t  with a state s of its own per request."""
+
+        def __init__(self, params, dtype, device):
+            super().__init__(dtype, device)
+            self.hidden, self.width = params["hidden_size"], params["state_size"]
+
+        def state_need(self):
+            return StateNeed((self.width,), torch.float32)
+
+        def param_specs(self):
+            return {"a": ParamSpec((self.width,), "vector"), "B.weight": ParamSpec((self.width, self.hidden)),
+                    "C.weight": ParamSpec((self.hidden, self.width))}
+
+        def load(self, tensors):
+            self.a, self.B, self.C = torch.sigmoid(tensors["a"]), tensors["B.weight"].float(), tensors["C.weight"].float()
+
+        def forward(self, x, step, slot):
+            u = x.float() @ self.B.T
+            out = torch.empty_like(u)
+            for r, slot_id in enumerate(step.req_slots_host):
+                s = slot.state[slot_id]
+                for n in range(step.cu_q_host[r], step.cu_q_host[r + 1]):
+                    s = self.a * s + u[n]
+                    out[n] = s
+                slot.state[slot_id] = s
+            return (out @ self.C.T).to(torch.float32)
+
+    class RoutedFeedForward(FeedForward):
+        """Two experts of one matrix each; a token goes to the expert its router logit favours."""
+
+        def __init__(self, params, dtype, device):
+            super().__init__(dtype, device)
+            self.hidden = params["hidden_size"]
+
+        def param_specs(self):
+            return {"router.weight": ParamSpec((2, self.hidden)), "experts.0.weight": ParamSpec((self.hidden, self.hidden)),
+                    "experts.1.weight": ParamSpec((self.hidden, self.hidden))}
+
+        def load(self, tensors):
+            self.t = {k: v.float() for k, v in tensors.items()}
+
+        def forward(self, x, step):
+            xf = x.float()
+            pick = (xf @ self.t["router.weight"].T).argmax(-1)
+            y0, y1 = xf @ self.t["experts.0.weight"].T, xf @ self.t["experts.1.weight"].T
+            return torch.where(pick[:, None] == 0, y0, y1)
+
+    class HalfSpeedRoPE(PositionEncoding):
+        """1-D rotation on row 2 of the positions with halved frequencies, first half of the head only."""
+        num_rows = 3
+
+        def __init__(self, params, dtype, device):
+            super().__init__(dtype, device)
+            self.theta = params["theta"]
+
+        def rotary_tables(self, head_dim):
+            rot = head_dim // 2
+            inv = 0.5 * plain_inv_freq(rot, self.theta)
+            return inv.to(self.device), torch.full((rot // 2,), 2, dtype=torch.int32, device=self.device)
+
+    register_part("mixer", "toy_decay", DecayMixer)
+    register_part("ffn", "toy_routed", RoutedFeedForward)
+    register_part("position", "toy_half_speed", HalfSpeedRoPE)
+
+
+def _plain_toy_model(model, toks, pos_row2):
+    """The toy model of `test_toy_parts...` computed whole, in plain float32 on the CPU."""
+    w = {}
+    for part, names in model.part_groups():
+        pass
+    hidden = model.spec.hidden_size
+    emb = model.embed.float().cpu()
+    h = emb[torch.tensor(toks)]
+    t = len(toks)
+    for block in model.blocks:
+        x = plain_rmsnorm(h, block.norm1.weight.cpu(), 1e-6)
+        m = block.mixer
+        if hasattr(m, "B"):
+            a, B, C = m.a.cpu(), m.B.cpu(), m.C.cpu()
+            s, ys = torch.zeros(B.shape[0]), []
+            for n in range(t):
+                s = a * s + B @ x[n]
+                ys.append(s)
+            y = torch.stack(ys) @ C.T
+        else:
+            nw = {k: v.float().cpu() for k, v in m.named_weights().items()}
+            q = (x @ nw["q_proj.weight"].T).view(t, m.nq, m.hd).transpose(0, 1)
+            k = (x @ nw["k_proj.weight"].T).view(t, m.nkv, m.hd).transpose(0, 1)
+            v = (x @ nw["v_proj.weight"].T).view(t, m.nkv, m.hd).transpose(0, 1)
+            rot = m.hd // 2
+            inv = 0.5 * plain_inv_freq(rot, 50.0)
+            ang = pos_row2.float()[:, None] * inv[None]
+            cos, sin = ang.cos(), ang.sin()
+
+            def rotate(z):
+                z = z.clone()
+                a1, a2 = z[..., :rot // 2].clone(), z[..., rot // 2:rot].clone()
+                z[..., :rot // 2] = a1 * cos - a2 * sin
+                z[..., rot // 2:rot] = a2 * cos + a1 * sin
+                return z
+
+            o = plain_attention(rotate(q), rotate(k), v, m.hd ** -0.5, m.window)
+            y = o.transpose(0, 1).reshape(t, m.nq * m.hd) @ nw["o_proj.weight"].T
+        h = h + y
+        x2 = plain_rmsnorm(h, block.norm2.weight.cpu(), 1e-6)
+        f = block.ffn
+        if hasattr(f, "t"):
+            tt = {k: v.cpu() for k, v in f.t.items()}
+            pick = (x2 @ tt["router.weight"].T).argmax(-1)
+            y2 = torch.where(pick[:, None] == 0, x2 @ tt["experts.0.weight"].T, x2 @ tt["experts.1.weight"].T)
+        else:
+            nw = {k: v.float().cpu() for k, v in f.named_weights().items()}
+            y2 = (torch.nn.functional.silu(x2 @ nw["gate_proj.weight"].T) * (x2 @ nw["up_proj.weight"].T)) @ nw["down_proj.weight"].T
+        h = h + y2
+    return plain_rmsnorm(h, model.final_norm.weight.cpu(), 1e-6) @ emb.T
+
+
+def test_toy_parts_register_build_and_step():
+    """A mixer with a state of its own, a routed feed-forward and another position encoding, all
+    defined above, in one model with a windowed attention layer: whole, cut into portions, and two
+    requests interleaved (so that each one's state must live in its own slot)."""
+    from qwen25vl_lite_amd.engine import StepEntry
+    from qwen25vl_lite_amd.parts import PartSpec
+    _register_toys()
+    hidden = 24
+    toy_pos = PartSpec("toy_half_speed", {"theta": 50.0})
+    decay = PartSpec("toy_decay", {"hidden_size": hidden, "state_size": 10})
+    routed = PartSpec("toy_routed", {"hidden_size": hidden})
+    swiglu = PartSpec("swiglu", {"hidden_size": hidden, "intermediate_size": 40})
+    layers = [(decay, routed), (_attn_spec(hidden, 3, 1, 8, toy_pos, window=9), swiglu), (decay, swiglu)]
+    model = _spec_model(layers, hidden, 40, seed=5)
+    assert [s is not None for s in model.entry_state] == [True, False, True]
+    assert "blocks.0.mix.B.weight" in model.expected_tensors() and "blocks.0.ff.router.weight" in model.expected_tensors()
+    runner = _runner(model, pages=8)
+    g = torch.Generator().manual_seed(9)
+    ta = torch.randint(0, 40, (30,), generator=g).tolist()
+    tb = torch.randint(0, 40, (21,), generator=g).tolist()
+    want_a = _plain_toy_model(model, ta, torch.arange(30))
+    want_b = _plain_toy_model(model, tb, torch.arange(21))
+    assert torch.allclose(_run(runner, "a", ta, [30]), want_a, atol=2e-4)
+    assert torch.allclose(_run(runner, "a2", ta, [4, 2, 11, 1, 1, 1, 10]), want_a, atol=2e-4)
+    # interleaved: portions of a beside single tokens of b, in the same steps
+    runner.admit("a")
+    runner.admit("b")
+    got_a, got_b, ia, ib = [], [], 0, 0
+    while ia < len(ta) or ib < len(tb):
+        entries = []
+        if ia < len(ta):
+            n = min(5, len(ta) - ia)
+            entries.append(StepEntry("a", ta[ia:ia + n], ia, want=list(range(n))))
+        if ib < len(tb):
+            entries.append(StepEntry("b", tb[ib:ib + 1], ib, want=[0]))
+        out = runner.execute(entries).cpu()
+        if ia < len(ta):
+            got_a.append(out[:n]); out = out[n:]; ia += n
+        if ib < len(tb):
+            got_b.append(out); ib += 1
+    assert torch.allclose(torch.cat(got_a), want_a, atol=2e-4) and torch.allclose(torch.cat(got_b), want_b, atol=2e-4)
+    # a slot that is taken again starts from a cleared state
+    runner.release("a"); runner.release("b")
+    assert torch.allclose(_run(runner, "again", tb, [21]), want_b, atol=2e-4)

@@ -3,7 +3,7 @@
 import pytest
 import torch
 
-from plain_model import plain_model_logits
+from plain_model import as_bfloat16, plain_model_logits
 from replay_util import (mixed_trace, portion_trace, random_tokens, round64, run_steps, tail_trace, whole_trace)
 
 pytestmark = pytest.mark.gpu
@@ -13,14 +13,20 @@ VOCAB = {"A": 256, "B": 509, "C": 300}
 
 
 def _requests(name):
+    name = name[0]
     return {f"r{i}": random_tokens(n, VOCAB[name], 100 * ord(name) + i) for i, n in enumerate(LENGTHS[name])}
 
 
-def _reference(model_dir, requests):
-    return {rid: plain_model_logits(model_dir, toks) for rid, toks in requests.items()}
+def _reference(model_dir, requests, dtype="float32"):
+    """float32 runs are held to the plain implementation as it is.  bfloat16 runs are held to the
+    plain implementation with its stored activations rounded to bfloat16 (the arithmetic stays
+    float32): that is the result a bfloat16 run should give, and it can be held to it tightly even
+    where peaked attention turns rounding into percents of a logit."""
+    store = as_bfloat16 if dtype == "bfloat16" else (lambda x: x)
+    return {rid: plain_model_logits(model_dir, toks, store=store) for rid, toks in requests.items()}
 
 
-def _compare(got, ref, dtype, what):
+def _compare(got, ref, dtype, what, bound=None):
     worst = 0.0
     for (rid, pos), row in got.items():
         want = ref[rid][pos]
@@ -29,10 +35,10 @@ def _compare(got, ref, dtype, what):
             ok = torch.allclose(row, want, atol=1e-4, rtol=1e-3)
             err = (row - want).abs().max().item()
         else:
-            # bfloat16: worst error against the largest logit, as the reference checks its fused
-            # kernel (reference src/qwen25vl_lite/paged_attn_triton.py:253)
+            # bfloat16: worst error against the largest logit, the measure the reference uses for
+            # its fused kernel (reference src/qwen25vl_lite/paged_attn_triton.py:253, bound 2e-2)
             err = ((row - want).abs().max() / want.abs().max()).item()
-            ok = err < 2e-2
+            ok = err < (bound or 2e-2)
         worst = max(worst, err)
         assert ok, f"{what}: request {rid} position {pos}: error {err:.3e}"
     return worst
@@ -44,17 +50,20 @@ def _replayer(model_dir, dtype, max_tokens):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "A_sharp", "B_sharp", "C_sharp"])
 def test_replay_every_way(model_dirs, name, dtype):
     d = model_dirs[name]
     requests = _requests(name)
-    ref = _reference(d, requests)
+    ref = _reference(d, requests, dtype)
     total = sum(len(t) for t in requests.values())
 
-    rp = _replayer(d, dtype, round64(max(LENGTHS[name])))
+    rp = _replayer(d, dtype, round64(max(LENGTHS[name[0]])))
     got = run_steps(rp, whole_trace(requests))
     assert len(got) == total
     print(name, dtype, "whole", _compare(got, ref, dtype, "whole"))
+    if dtype == "bfloat16" and "sharp" not in name:
+        # against pure float32 arithmetic the reference's bound for reduced precision holds
+        print(name, "bfloat16 against float32", _compare(got, _reference(d, requests), dtype, "whole/float32"))
     assert rp.runner.cache.pages_in_use() == [0] * len(rp.runner.cache.groups)
 
     got = run_steps(rp, tail_trace(requests))
