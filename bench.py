@@ -1,0 +1,188 @@
+"""Decode and prefill throughput of the engine on one MI355X.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+The model has the layer sizes of BASELINE.json's configs[2] (the Qwen2.5-VL-7B text decoder)
+with random weights N(0, 0.02) in bfloat16; token ids are seeded uniform random integers.  A
+"step" is one decode step of the scheduler: every live request gets its next token through the
+engine's own path (batch building, the step function over the paged cache, sampling on the
+device, the copy of the sampled ids to the host).  The default batch is 8 requests with
+512-token prompts.  The same run also measures decoding at batch 1 and 64 and a 2,048-token
+prefill, and prints one JSON line.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
+MFMA_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+
+def seven_b_config(layers=None):
+    """configs[2] of BASELINE.json as a config.json dictionary."""
+    raw = {
+        "architectures": ["Qwen2_5_VLForConditionalGeneration"], "model_type": "qwen2_5_vl",
+        "tie_word_embeddings": False, "hidden_size": 3584, "intermediate_size": 18944,
+        "num_hidden_layers": 28, "num_attention_heads": 28, "num_key_value_heads": 4, "vocab_size": 152064,
+        "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "sliding_window": 32768, "use_sliding_window": False,
+        "max_position_embeddings": 8192, "rope_scaling": {"type": "mrope", "mrope_section": [16, 24, 24]},
+    }
+    if layers:
+        raw["num_hidden_layers"] = int(layers)
+    return raw
+
+
+def step_bytes(t, batch, ctx, bytes_per_value=2):
+    """Bytes a decode step has to read: every weight it uses once (all layers and the head; of the
+    embedding only the rows looked up) and the keys and values of the live requests."""
+    h, hd, inter = t.hidden_size, t.head_dim, t.intermediate_size
+    nh, nkv = t.num_attention_heads, t.num_key_value_heads
+    per_layer = h * (nh + 2 * nkv) * hd + nh * hd * h + 3 * h * inter
+    weights = (per_layer * t.num_hidden_layers + t.vocab_size * h) * bytes_per_value
+    kv = batch * ctx * t.kv_bytes_per_token(bytes_per_value)
+    return weights + kv
+
+
+def prefill_flops(t, tokens):
+    h, hd, inter = t.hidden_size, t.head_dim, t.intermediate_size
+    nh, nkv = t.num_attention_heads, t.num_key_value_heads
+    per_layer = h * (nh + 2 * nkv) * hd + nh * hd * h + 3 * h * inter
+    linear = 2.0 * tokens * per_layer * t.num_hidden_layers
+    attention = 4.0 * nh * hd * (tokens * (tokens + 1) / 2) * t.num_hidden_layers   # causal: QK^T and PV
+    head = 2.0 * t.vocab_size * h                                                   # one row
+    return linear + attention + head
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--prompt-tokens", type=int, default=512)
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration has")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and the prefill")
+    ap.add_argument("--no-graph", action="store_true", help="do not replay decode steps from a HIP graph")
+    args = ap.parse_args(argv)
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print(f"bench.py measures one GPU: this engine does not run on {args.gpus} GPUs (run with --gpus 1)")
+        return 2
+
+    import torch
+
+    from qwen25vl_lite_amd import EngineConfig, LLMEngine, ModelRunner, Qwen25VLConfig, SamplingParams, build_model
+    from qwen25vl_lite_amd.config import dtype_from_name
+    from qwen25vl_lite_amd.weights import fill_random
+
+    cfg = Qwen25VLConfig.from_dict(seven_b_config(args.layers))
+    t = cfg.text_config
+    dtype = dtype_from_name(args.dtype)
+    model = build_model(cfg, dtype, "cuda:0")
+    fill_random(model, seed=0)
+    torch.cuda.synchronize()
+
+    page = 16
+    max_ctx = 8192
+    gen = torch.Generator().manual_seed(0)
+
+    def make_engine(max_seqs, tokens_per_seq, budget):
+        ecfg = EngineConfig(num_blocks=max_seqs * ((tokens_per_seq + page - 1) // page + 1), block_size=page,
+                            max_num_seqs=max_seqs, max_num_batched_tokens=budget, max_model_len=max_ctx,
+                            enable_prefix_cache=False, dtype=dtype, device="cuda:0", hip_graph=not args.no_graph)
+        runner = ModelRunner(model, ecfg)
+        return LLMEngine(runner, ecfg), runner
+
+    def prompt(n):
+        return torch.randint(0, t.vocab_size, (n,), generator=gen).tolist()
+
+    def decode_rate(batch, steps, warmup):
+        budget = max(4096, batch)
+        # requests admitted first already decode while later prompts are still prefilled
+        early = (batch * args.prompt_tokens + budget - 1) // budget + 2
+        total = args.prompt_tokens + warmup + steps + early + 2
+        engine, runner = make_engine(batch, total, budget)
+        params = SamplingParams(temperature=0.0, max_tokens=warmup + steps + early + 1, ignore_eos=True)
+        for _ in range(batch):
+            engine.add_request(prompt(args.prompt_tokens), params)
+        while any(s.remaining > 1 for s in engine.running) or engine.waiting:
+            engine.step()                      # prefill
+        for _ in range(warmup):
+            engine.step()
+        torch.cuda.synchronize()
+        before = engine.stats_.decode_tokens
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            engine.step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        tokens = engine.stats_.decode_tokens - before
+        assert tokens == batch * steps, (tokens, batch, steps)
+        ctx_mid = args.prompt_tokens + warmup + steps // 2
+        del engine, runner
+        torch.cuda.empty_cache()
+        return tokens / dt, dt / steps * 1e3, ctx_mid
+
+    def prefill_rate(tokens, reps=3):
+        engine, runner = make_engine(2, tokens + 8, tokens)
+        params = SamplingParams(temperature=0.0, max_tokens=1, ignore_eos=True)
+        times = []
+        for i in range(reps + 1):
+            engine.add_request(prompt(tokens), params)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            done = engine.step()               # the whole prompt in one step, then its first token is sampled
+            torch.cuda.synchronize()
+            assert len(done) == 1
+            if i:
+                times.append(time.perf_counter() - t0)
+        del engine, runner
+        torch.cuda.empty_cache()
+        return min(times)
+
+    value, ms_per_step, ctx_mid = decode_rate(args.batch, args.steps, args.warmup)
+    need = step_bytes(t, args.batch, ctx_mid, 2 if args.dtype == "bfloat16" else 4)
+    achieved = need / (ms_per_step * 1e-3) / 1e9
+    peak_key = "bf16" if args.dtype == "bfloat16" else "fp32"
+    line = {
+        "metric": "decode tok/s (Qwen2.5-VL-7B text decoder, bf16, batch 8, 512-token prompts)",
+        "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
+        "config": {
+            "model": "Qwen2.5-VL-7B text decoder (random weights)", "layers": t.num_hidden_layers,
+            "layers_of_config": 28, "hidden_size": t.hidden_size, "heads": t.num_attention_heads,
+            "kv_heads": t.num_key_value_heads, "head_dim": t.head_dim, "intermediate_size": t.intermediate_size,
+            "vocab_size": t.vocab_size, "global_batch": args.batch, "seq_len": args.prompt_tokens,
+            "context_mid": ctx_mid, "max_context": max_ctx, "page_size": page, "parallelism": "single GPU",
+            "hip_graph": not args.no_graph,
+        },
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+    }
+    if not args.no_points:
+        points = {}
+        for b, steps in ((1, min(args.steps, 64)), (64, min(args.steps, 64))):
+            rate, _, _ = decode_rate(b, steps, min(args.warmup, 4))
+            points[f"decode_b{b}"] = round(rate, 2)
+        line["points"] = points
+        tokens = 2048
+        sec = prefill_rate(tokens)
+        flops = prefill_flops(t, tokens)
+        line["prefill"] = {"value": round(tokens / sec, 1), "tokens": tokens, "ms": round(sec * 1e3, 3),
+                           "frac": round(flops / sec / MFMA_PEAK[peak_key], 4)}
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    raise SystemExit(main())
