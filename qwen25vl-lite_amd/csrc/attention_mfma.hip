@@ -1,0 +1,321 @@
+// Paged attention on the matrix cores: bfloat16 storage, head size HD (a multiple of 16, set at
+// compile time with -DHD=...), float32 softmax.  One kernel serves prompt portions and decoded
+// tokens of a mixed batch.
+//
+// Work is cut into tiles of 16 "columns" of one request and one key/value head.  A column is a
+// (token of this step, query head of the group) pair, token-major, so the group's heads share
+// every key and value that is loaded.  One wave owns a tile and walks the request's keys in
+// blocks of 32 by absolute index, with two kinds of v_mfma_f32_16x16x32_bf16 per block:
+//
+//   S^T[key, col]  = K[key, :] . Q[col, :]        A = keys x dims,   B = dims x columns
+//   O^T[dim, col] += V^T[dim, key] . P^T[key, col] A = dims x keys,   B = keys x columns
+//
+// Computing the transposes keeps a column in one lane (lane % 16) through both products: the
+// softmax statistics of a column live in that lane, and the probabilities come out of the first
+// product in the register layout the second wants as its B operand, if the 16 rows of the two
+// key blocks are permuted so that lane group g = lane / 16 ends up with the 8 consecutive keys
+// 8g .. 8g+7.  Keys are stored [page][kv head][slot][HD] and values transposed,
+// [page][kv head][HD][slot], so both A operands are plain 16-byte loads from the pages.
+//
+// With SPLIT, a tile's keys are divided among `nsplit` waves; each writes its unnormalised sums
+// and statistics to a scratch buffer and a second kernel merges them (decode with long contexts
+// and few requests).
+#include "common.h"
+
+#ifndef HD
+#error "compile with -DHD=<head size>"
+#endif
+#if HD % 16 != 0 || HD < 16 || HD > 256
+#error "HD must be a multiple of 16 between 16 and 256"
+#endif
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+#define KS ((HD + 31) / 32)  // 32-wide steps over the head for Q.K
+#define NT (HD / 16)         // 16-wide tiles of the head for P.V
+#define LOG2E 1.4426950408889634f
+
+__device__ __forceinline__ bf16x8_t load8(const bf16_t* p) {
+  return __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(p));
+}
+__device__ __forceinline__ bf16x8_t zero8() {
+  u32x4_t z = {0u, 0u, 0u, 0u};
+  return __builtin_bit_cast(bf16x8_t, z);
+}
+__device__ __forceinline__ uint32_t pack2(float a, float b) {
+  return (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
+}
+
+struct TileState {
+  float m, l;
+  f32x4_t acc[NT];
+};
+
+// Walk keys [key_begin, key_end] (inclusive, absolute) of one tile.
+__device__ __forceinline__ void attend(const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
+                                       const int* __restrict__ bt, int table_width, int nkv, int kvh, int ps,
+                                       const bf16x8_t* qb, int my_lo, int my_p, float scale_log2, int key_begin,
+                                       int key_end, TileState& st) {
+  const int lane = threadIdx.x & 63, lg = lane >> 4, r = lane & 15;
+  const int max_key = table_width * ps - 1;
+  for (int kb = key_begin >> 5; (kb << 5) <= key_end; ++kb) {
+    const int key0 = kb << 5;
+    // ---- S^T = K . Q^T for two blocks of 16 rows; row r of block b holds key 8*(r/4) + 4b + r%4
+    f32x4_t s[2];
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const int key = key0 + 8 * (r >> 2) + 4 * b + (r & 3);
+      int page = bt[min(key, max_key) / ps];
+      page = page < 0 ? 0 : page;
+      const bf16_t* krow = kc + (((size_t)page * nkv + kvh) * ps + (size_t)(key % ps)) * HD;
+      f32x4_t a = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const int d = ks * 32 + 8 * lg;
+        const bf16x8_t kk = (d < HD) ? load8(krow + d) : zero8();
+        a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kk, qb[ks], a, 0, 0, 0);
+      }
+      s[b] = a;
+    }
+    // ---- mask and online softmax; this lane holds keys key0 + 8*lg + j of column r
+    float sv[8];
+    float mloc = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int key = key0 + 8 * lg + j;
+      const float raw = (j < 4) ? s[0][j] : s[1][j - 4];
+      const bool ok = key >= my_lo && key <= my_p && key >= key_begin && key <= key_end;
+      sv[j] = ok ? raw * scale_log2 : -INFINITY;
+      mloc = fmaxf(mloc, sv[j]);
+    }
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 16, QVL_WAVE));
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, QVL_WAVE));
+    const float m_new = fmaxf(st.m, mloc);
+    float alpha = 1.f, psum = 0.f;
+    float pv[8];
+    if (m_new == -INFINITY) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) pv[j] = 0.f;
+    } else {
+      alpha = exp2f(st.m - m_new);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        pv[j] = exp2f(sv[j] - m_new);
+        psum += pv[j];
+      }
+    }
+    psum += __shfl_xor(psum, 16, QVL_WAVE);
+    psum += __shfl_xor(psum, 32, QVL_WAVE);
+    st.l = st.l * alpha + psum;
+    st.m = m_new;
+    u32x4_t packed = {pack2(pv[0], pv[1]), pack2(pv[2], pv[3]), pack2(pv[4], pv[5]), pack2(pv[6], pv[7])};
+    const bf16x8_t pb = __builtin_bit_cast(bf16x8_t, packed);
+    // ---- O^T += V^T . P^T; this lane reads keys key0 + 8*lg .. +7 of channel dt*16 + r
+    const int vkey = key0 + 8 * lg;
+    int vpage = bt[min(vkey, max_key) / ps];
+    vpage = (vpage < 0 || vkey > max_key) ? 0 : vpage;
+    const bf16_t* vbase = vc + (((size_t)vpage * nkv + kvh) * HD) * ps + (size_t)(vkey % ps);
+#pragma unroll
+    for (int dt = 0; dt < NT; ++dt) {
+      const bf16x8_t vv = load8(vbase + (size_t)(dt * 16 + r) * ps);
+      f32x4_t o = st.acc[dt];
+      o[0] *= alpha; o[1] *= alpha; o[2] *= alpha; o[3] *= alpha;
+      st.acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv, pb, o, 0, 0, 0);
+    }
+  }
+}
+
+// Everything a wave needs to know about its tile.
+struct TileInfo {
+  bool valid;      // this lane's column exists
+  int token;       // row of q / out
+  int head;        // query head
+  int my_lo, my_p; // first and last key this lane's column sees
+  int lo_tile, hi_tile;
+};
+
+__device__ __forceinline__ TileInfo tile_info(const int* cu_q, const int* ctx_len, int r, int ct, int g, int kvh,
+                                              int window) {
+  const int lane = threadIdx.x & 63, c = lane & 15;
+  const int q0 = cu_q[r], qlen = cu_q[r + 1] - q0, ctx = ctx_len[r];
+  const int col = ct * 16 + c;
+  const int i = col / g, gh = col - i * g;
+  TileInfo t;
+  t.valid = i < qlen;
+  t.token = q0 + (t.valid ? i : 0);
+  t.head = kvh * g + gh;
+  const int p = ctx - qlen + (t.valid ? i : 0);
+  t.my_p = t.valid ? p : -1;
+  t.my_lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  const int i_first = (ct * 16) / g;
+  int i_last = (ct * 16 + 15) / g;
+  i_last = i_last < qlen - 1 ? i_last : qlen - 1;
+  const int p_first = ctx - qlen + i_first;
+  t.lo_tile = (window > 0 && p_first - window + 1 > 0) ? p_first - window + 1 : 0;
+  t.hi_tile = ctx - qlen + i_last;
+  return t;
+}
+
+__device__ __forceinline__ void load_q(const bf16_t* __restrict__ q, int nq, const TileInfo& t, bf16x8_t* qb) {
+  const int lg = (threadIdx.x & 63) >> 4;
+  const bf16_t* qrow = q + ((size_t)t.token * nq + t.head) * HD;
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    const int d = ks * 32 + 8 * lg;
+    qb[ks] = (t.valid && d < HD) ? load8(qrow + d) : zero8();
+  }
+}
+
+__global__ __launch_bounds__(256) void attn_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc,
+                                                        const bf16_t* __restrict__ vc, const int* __restrict__ bt,
+                                                        int table_width, const int* __restrict__ cu_q,
+                                                        const int* __restrict__ ctx_len,
+                                                        const int* __restrict__ tile_req,
+                                                        const int* __restrict__ tile_ct, int num_tiles,
+                                                        bf16_t* __restrict__ out, int nq, int nkv, int ps, int window,
+                                                        float scale) {
+  const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (item >= num_tiles) return;
+  const int kvh = blockIdx.y, g = nq / nkv;
+  const int r = tile_req[item], ct = tile_ct[item];
+  const TileInfo t = tile_info(cu_q, ctx_len, r, ct, g, kvh, window);
+  bf16x8_t qb[KS];
+  load_q(q, nq, t, qb);
+  TileState st;
+  st.m = -INFINITY;
+  st.l = 0.f;
+#pragma unroll
+  for (int dt = 0; dt < NT; ++dt) st.acc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  attend(kc, vc, bt + (size_t)r * table_width, table_width, nkv, kvh, ps, qb, t.my_lo, t.my_p, scale * LOG2E,
+         t.lo_tile, t.hi_tile, st);
+  if (!t.valid) return;
+  const int lg = (threadIdx.x & 63) >> 4;
+  const float inv = 1.0f / st.l;
+  bf16_t* orow = out + ((size_t)t.token * nq + t.head) * HD;
+#pragma unroll
+  for (int dt = 0; dt < NT; ++dt) {
+    const int d = dt * 16 + 4 * lg;
+    uint2 w;
+    w.x = pack2(st.acc[dt][0] * inv, st.acc[dt][1] * inv);
+    w.y = pack2(st.acc[dt][2] * inv, st.acc[dt][3] * inv);
+    *reinterpret_cast<uint2*>(orow + d) = w;
+  }
+}
+
+// ---- split over keys: partial sums to scratch, then a merge ---------------------------------
+// scratch layout per (tile, kv head, split): 16 columns x PART_COLS floats (HD sums, m, l, and
+// padding that keeps every column 16-byte aligned).
+#define PART_COLS (HD + 4)
+#define PART_STRIDE (16 * PART_COLS)
+
+__global__ __launch_bounds__(256) void attn_mfma_split_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
+    const int* __restrict__ bt, int table_width, const int* __restrict__ cu_q, const int* __restrict__ ctx_len,
+    const int* __restrict__ tile_req, const int* __restrict__ tile_ct, int num_tiles, float* __restrict__ scratch,
+    int nq, int nkv, int ps, int window, float scale, int nsplit, int keys_per_split) {
+  const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (item >= num_tiles * nsplit) return;
+  const int tile = item / nsplit, split = item - tile * nsplit;
+  const int kvh = blockIdx.y, g = nq / nkv;
+  const int r = tile_req[tile], ct = tile_ct[tile];
+  const TileInfo t = tile_info(cu_q, ctx_len, r, ct, g, kvh, window);
+  // splits are cut by absolute key index, in multiples of 32
+  const int first = (t.lo_tile >> 5 << 5) + split * keys_per_split;
+  int last = first + keys_per_split - 1;
+  last = last < t.hi_tile ? last : t.hi_tile;
+  TileState st;
+  st.m = -INFINITY;
+  st.l = 0.f;
+#pragma unroll
+  for (int dt = 0; dt < NT; ++dt) st.acc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  if (first <= last) {
+    bf16x8_t qb[KS];
+    load_q(q, nq, t, qb);
+    attend(kc, vc, bt + (size_t)r * table_width, table_width, nkv, kvh, ps, qb, t.my_lo, t.my_p, scale * LOG2E,
+           first, last, st);
+  }
+  const int lane = threadIdx.x & 63, lg = lane >> 4, c = lane & 15;
+  float* part = scratch + (((size_t)tile * nkv + kvh) * nsplit + split) * PART_STRIDE + (size_t)c * PART_COLS;
+#pragma unroll
+  for (int dt = 0; dt < NT; ++dt) {
+    const int d = dt * 16 + 4 * lg;
+    *reinterpret_cast<float4*>(part + d) = float4{st.acc[dt][0], st.acc[dt][1], st.acc[dt][2], st.acc[dt][3]};
+  }
+  if (lg == 0) {
+    part[HD] = st.m;
+    part[HD + 1] = st.l;
+  }
+}
+
+__global__ void attn_mfma_merge_kernel(const float* __restrict__ scratch, const int* __restrict__ cu_q,
+                                       const int* __restrict__ tile_req, const int* __restrict__ tile_ct,
+                                       bf16_t* __restrict__ out, int nq, int nkv, int nsplit) {
+  // one block per (tile, kv head); thread = (column, channel group)
+  const int tile = blockIdx.x, kvh = blockIdx.y, g = nq / nkv;
+  const int r = tile_req[tile], ct = tile_ct[tile];
+  const int q0 = cu_q[r], qlen = cu_q[r + 1] - q0;
+  const float* base = scratch + ((size_t)tile * nkv + kvh) * nsplit * PART_STRIDE;
+  for (int idx = threadIdx.x; idx < 16 * HD; idx += blockDim.x) {
+    const int c = idx / HD, d = idx - c * HD;
+    const int col = ct * 16 + c;
+    const int i = col / g, gh = col - i * g;
+    if (i >= qlen) continue;
+    float m = -INFINITY;
+    for (int s = 0; s < nsplit; ++s) m = fmaxf(m, base[(size_t)s * PART_STRIDE + c * PART_COLS + HD]);
+    float num = 0.f, den = 0.f;
+    for (int s = 0; s < nsplit; ++s) {
+      const float* p = base + (size_t)s * PART_STRIDE + c * PART_COLS;
+      const float w = (p[HD] == -INFINITY) ? 0.f : exp2f(p[HD] - m);
+      num += w * p[d];
+      den += w * p[HD + 1];
+    }
+    out[((size_t)(q0 + i) * nq + kvh * g + gh) * HD + d] = f32_to_bf16(num / den);
+  }
+}
+
+static int check_common(int num_tiles, int nq, int nkv, int ps, int table_width) {
+  if (num_tiles <= 0) return QVL_OK;
+  if (nq <= 0 || nkv <= 0 || nq % nkv || ps <= 0 || ps % 16 || table_width <= 0) return QVL_ERR_SHAPE;
+  if (nkv > 65535) return QVL_ERR_LIMIT;
+  return -1;
+}
+
+extern "C" int qvl_attn_mfma_head_dim() { return HD; }
+
+extern "C" int qvl_attn_mfma(const void* q, const void* kc, const void* vc, const void* bt, int table_width,
+                             const void* cu_q, const void* ctx_len, const void* tile_req, const void* tile_ct,
+                             int num_tiles, void* out, int nq, int nkv, int ps, int window, float scale,
+                             hipStream_t stream) {
+  const int c = check_common(num_tiles, nq, nkv, ps, table_width);
+  if (c >= 0) return c;
+  const dim3 grid((num_tiles + 3) / 4, nkv);
+  hipLaunchKernelGGL(attn_mfma_kernel, grid, dim3(256), 0, stream, (const bf16_t*)q, (const bf16_t*)kc,
+                     (const bf16_t*)vc, (const int*)bt, table_width, (const int*)cu_q, (const int*)ctx_len,
+                     (const int*)tile_req, (const int*)tile_ct, num_tiles, (bf16_t*)out, nq, nkv, ps, window, scale);
+  return qvl_launch_status();
+}
+
+// Floats the scratch buffer of a split call must hold.
+extern "C" long long qvl_attn_mfma_scratch_floats(int num_tiles, int nkv, int nsplit) {
+  return (long long)num_tiles * nkv * nsplit * PART_STRIDE;
+}
+
+extern "C" int qvl_attn_mfma_split(const void* q, const void* kc, const void* vc, const void* bt, int table_width,
+                                   const void* cu_q, const void* ctx_len, const void* tile_req, const void* tile_ct,
+                                   int num_tiles, void* out, void* scratch, int nq, int nkv, int ps, int window,
+                                   float scale, int nsplit, int keys_per_split, hipStream_t stream) {
+  const int c = check_common(num_tiles, nq, nkv, ps, table_width);
+  if (c >= 0) return c;
+  if (nsplit <= 0 || keys_per_split <= 0 || keys_per_split % 32) return QVL_ERR_SHAPE;
+  const dim3 grid((num_tiles * nsplit + 3) / 4, nkv);
+  hipLaunchKernelGGL(attn_mfma_split_kernel, grid, dim3(256), 0, stream, (const bf16_t*)q, (const bf16_t*)kc,
+                     (const bf16_t*)vc, (const int*)bt, table_width, (const int*)cu_q, (const int*)ctx_len,
+                     (const int*)tile_req, (const int*)tile_ct, num_tiles, (float*)scratch, nq, nkv, ps, window,
+                     scale, nsplit, keys_per_split);
+  if (hipGetLastError() != hipSuccess) return QVL_ERR_LAUNCH;
+  hipLaunchKernelGGL(attn_mfma_merge_kernel, dim3(num_tiles, nkv), dim3(256), 0, stream, (const float*)scratch,
+                     (const int*)cu_q, (const int*)tile_req, (const int*)tile_ct, (bf16_t*)out, nq, nkv, nsplit);
+  return qvl_launch_status();
+}

@@ -1,15 +1,91 @@
-"""Dispatch to the matrix-core attention kernel (bfloat16, head sizes in steps of 16)."""
+"""Dispatch to the matrix-core attention kernel (bfloat16, head sizes in steps of 16).
+
+The kernel is compiled per head size (``-DHD=...``) at its first use.  A step's tokens are cut
+into tiles of 16 columns, a column being a (token, query head of one key/value group) pair; the
+tile list depends on the batch and on the group size only and is built once per step.
+"""
 
 from __future__ import annotations
 
-from typing import Optional
+import ctypes
+from typing import Optional, Tuple
 
+import numpy as np
 import torch
 
-__all__ = ["try_attention"]
+from .kernels import _check, _fn, _need, _ptr, _stream
+
+__all__ = ["try_attention", "supports", "tiles_for", "plan_splits"]
+
+_c_int, _c_float, _c_ptr = ctypes.c_int, ctypes.c_float, ctypes.c_void_p
+_MAX_HD = 256
+TARGET_WAVES = 1024      # enough waves to fill 256 compute units
+MIN_KEYS_PER_SPLIT = 64
+
+
+def supports(head_dim: int, dtype: torch.dtype) -> bool:
+    return dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= _MAX_HD
+
+
+def tiles_for(cu_q, group: int) -> Tuple[np.ndarray, np.ndarray]:
+    """``(tile_req, tile_ct)``: for request r with q tokens, ceil(q * group / 16) tiles."""
+    q = np.diff(np.asarray(cu_q, dtype=np.int64))
+    counts = (q * group + 15) // 16
+    req = np.repeat(np.arange(len(q), dtype=np.int32), counts)
+    starts = np.cumsum(counts) - counts
+    ct = (np.arange(int(counts.sum()), dtype=np.int64) - np.repeat(starts, counts)).astype(np.int32)
+    return req, ct
+
+
+def plan_splits(num_tiles: int, nkv: int, max_ctx: int) -> Tuple[int, int]:
+    """``(nsplit, keys_per_split)``; nsplit 1 means the unsplit kernel."""
+    waves = num_tiles * nkv
+    if waves >= TARGET_WAVES // 2 or max_ctx <= 2 * MIN_KEYS_PER_SPLIT:
+        return 1, 0
+    want = (TARGET_WAVES + waves - 1) // waves
+    per = max(MIN_KEYS_PER_SPLIT, ((max_ctx + want - 1) // want + 31) // 32 * 32)
+    nsplit = (max_ctx + 31 + per - 1) // per
+    return (nsplit, per) if nsplit > 1 else (1, 0)
+
+
+def _step_tiles(step, group: int, device):
+    cache = step.derived
+    key = ("tiles", group)
+    if key not in cache:
+        req, ct = tiles_for(step.cu_q_host, group)
+        both = torch.from_numpy(np.concatenate([req, ct])).to(device, non_blocking=True)
+        cache[key] = (both[:len(req)], both[len(req):], len(req))
+    return cache[key]
 
 
 def try_attention(q, k_cache, v_cache, block_table, step, num_q_heads: int, window: Optional[int],
                   scale: float) -> Optional[torch.Tensor]:
     """The attention through the matrix-core kernel, or None if it does not take this shape."""
-    return None
+    pages, nkv, ps, hd = k_cache.shape
+    if not supports(hd, q.dtype) or ps % 16:
+        return None
+    n, nq = q.shape[0], int(num_q_heads)
+    _need(q.is_cuda and q.shape == (n, nq * hd) and q.is_contiguous(), "q must be contiguous [N, nq hd] on the GPU")
+    _need(k_cache.dtype == v_cache.dtype == torch.bfloat16 and k_cache.is_contiguous() and v_cache.is_contiguous()
+          and tuple(v_cache.shape) == (pages, nkv, hd, ps), "cache must be bfloat16 [pages, nkv, ps, hd] / [.., hd, ps]")
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous()
+          and block_table.shape[0] == step.num_reqs, "block_table must be int32 [R, width]")
+    _need(nq % nkv == 0, "query heads must be a multiple of key/value heads")
+    tile_req, tile_ct, num_tiles = _step_tiles(step, nq // nkv, q.device)
+    out = torch.empty_like(q)
+    defines = {"HD": hd}
+    nsplit, per = plan_splits(num_tiles, nkv, step.max_ctx_len)
+    common = [_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(step.cu_q),
+              _ptr(step.ctx_len), _ptr(tile_req), _ptr(tile_ct), num_tiles, _ptr(out)]
+    if nsplit == 1:
+        fn = _fn("attention_mfma", "qvl_attn_mfma",
+                 [_c_ptr] * 4 + [_c_int] + [_c_ptr] * 4 + [_c_int, _c_ptr] + [_c_int] * 4 + [_c_float, _c_ptr], defines)
+        _check(fn(*common, nq, nkv, ps, int(window or 0), float(scale), _stream()), "paged_attention (matrix cores)")
+    else:
+        scratch = torch.empty(num_tiles * nkv * nsplit * 16 * (hd + 4), dtype=torch.float32, device=q.device)
+        fn = _fn("attention_mfma", "qvl_attn_mfma_split",
+                 [_c_ptr] * 4 + [_c_int] + [_c_ptr] * 4 + [_c_int, _c_ptr, _c_ptr] + [_c_int] * 4
+                 + [_c_float, _c_int, _c_int, _c_ptr], defines)
+        _check(fn(*common, _ptr(scratch), nq, nkv, ps, int(window or 0), float(scale), nsplit, per, _stream()),
+               "paged_attention (matrix cores, split)")
+    return out

@@ -14,6 +14,12 @@ LIBRARIES = [
     ("attention_generic", {}),
     ("gemm_f32", {}),
     ("sample", {}),
+    # the matrix-core attention is compiled per head size; these are the sizes the tests and the
+    # benchmark use, any other multiple of 16 is compiled at its first use
+    ("attention_mfma", {"HD": 128}),
+    ("attention_mfma", {"HD": 16}),
+    ("attention_mfma", {"HD": 48}),
+    ("attention_mfma", {"HD": 80}),
 ]
 
 

@@ -112,6 +112,7 @@ class StepContext:
     max_q_len: int = 0
     max_ctx_len: int = 0
     dtype: torch.dtype = torch.float32
+    derived: Dict[Any, Any] = field(default_factory=dict)   # per-step arrays kernels derive once (tile lists)
 
 
 @dataclass

@@ -115,22 +115,19 @@ def _paged(k, v, ps, pages, dtype, seed):
     return kc, vc, table
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("nq, nkv, hd, window", [(6, 2, 24, None), (5, 1, 48, 40), (8, 8, 16, 7), (14, 2, 128, None),
-                                                 (4, 2, 80, 130)])
-def test_paged_attention_generic(dtype, nq, nkv, hd, window):
+ATTN_SHAPES = [(6, 2, 24, None), (5, 1, 48, 40), (8, 8, 16, 7), (14, 2, 128, None), (4, 2, 80, 130)]
+
+
+def _attention_case(dtype, nq, nkv, hd, window):
     """Prompt portions and single tokens of several requests in one call, pages shuffled, stale
     values in every unused slot.  One query and one far key are scaled so that a single score
     dominates: a kernel that misses that key (a page, a window edge) fails by far."""
-    from qwen25vl_lite_amd.ops import kernels
     torch.manual_seed(nq * hd)
     ps = 16
     lens = [333, 17, 64, 1]           # context of each request after this step
     qlens = [5, 17, 1, 1]             # of which the last qlen are this step's tokens
-    k = [torch.randn(nkv, t, hd) for t in lens]
-    v = [torch.randn(nkv, t, hd) for t in lens]
-    k = [x.to(dtype).float() for x in k]
-    v = [x.to(dtype).float() for x in v]
+    k = [torch.randn(nkv, t, hd).to(dtype).float() for t in lens]
+    v = [torch.randn(nkv, t, hd).to(dtype).float() for t in lens]
     q_all = [torch.randn(nq, t, hd) for t in lens]
     far = 2 if window is None else max(0, 332 - window + 1)      # the first key the last query still sees
     kf = k[0][:, far].repeat_interleave(nq // nkv, 0)
@@ -146,16 +143,46 @@ def test_paged_attention_generic(dtype, nq, nkv, hd, window):
             req.append(r)
             seqpos.append(p)
             want.append(full[:, p].reshape(-1))
-    q = torch.stack(qs).to(dtype).cuda()
-    out = kernels.paged_attention_generic(q, kc.cuda(), vc.cuda(), table.cuda(),
-                                          torch.tensor(req, dtype=torch.int32).cuda(),
-                                          torch.tensor(seqpos, dtype=torch.int32).cuda(), nq, window, scale)
     want = torch.stack(want)
+    # the dominated row (request 0, position 332) really is the far key's value
+    assert torch.allclose(want[4].view(nq, hd), v[0][:, far].repeat_interleave(nq // nkv, 0), atol=1e-3)
+    return dict(q=torch.stack(qs).to(dtype).cuda(), kc=kc.cuda(), vc=vc.cuda(), table=table.cuda(),
+                req=torch.tensor(req, dtype=torch.int32).cuda(), seqpos=torch.tensor(seqpos, dtype=torch.int32).cuda(),
+                want=want, scale=scale, lens=lens, qlens=qlens)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq, nkv, hd, window", ATTN_SHAPES)
+def test_paged_attention_generic(dtype, nq, nkv, hd, window):
+    from qwen25vl_lite_amd.ops import kernels
+    c = _attention_case(dtype, nq, nkv, hd, window)
+    out = kernels.paged_attention_generic(c["q"], c["kc"], c["vc"], c["table"], c["req"], c["seqpos"], nq, window,
+                                          c["scale"])
     tol = dict(atol=2e-5, rtol=1e-4) if dtype == torch.float32 else dict(atol=1.5e-2, rtol=2e-2)
-    assert torch.allclose(out.float().cpu(), want, **tol), (out.float().cpu() - want).abs().max()
-    # the dominated row really is dominated by the far key's value
-    row = 4  # request 0, position 332
-    assert torch.allclose(want[row].view(nq, hd), v[0][:, far].repeat_interleave(nq // nkv, 0), atol=1e-3)
+    assert torch.allclose(out.float().cpu(), c["want"], **tol), (out.float().cpu() - c["want"]).abs().max()
+
+
+@pytest.mark.parametrize("split", [False, True])
+@pytest.mark.parametrize("nq, nkv, hd, window", [s for s in ATTN_SHAPES if s[2] % 16 == 0])
+def test_paged_attention_matrix_cores(nq, nkv, hd, window, split, monkeypatch):
+    """The matrix-core kernel on the same case, unsplit and with the keys split among waves."""
+    from qwen25vl_lite_amd.ops import attention_mfma
+    from qwen25vl_lite_amd.parts import StepContext
+    c = _attention_case(torch.bfloat16, nq, nkv, hd, window)
+    monkeypatch.setattr(attention_mfma, "plan_splits", (lambda t, n, m: (7, 64)) if split else (lambda t, n, m: (1, 0)))
+    cu = [0]
+    for ql in c["qlens"]:
+        cu.append(cu[-1] + ql)
+    none = torch.zeros(0, dtype=torch.int32).cuda()
+    step = StepContext(num_tokens=cu[-1], num_reqs=4, token_ids=none, positions=none, token_req=c["req"],
+                       token_seqpos=c["seqpos"], cu_q=torch.tensor(cu, dtype=torch.int32).cuda(),
+                       ctx_len=torch.tensor(c["lens"], dtype=torch.int32).cuda(), req_slots=none, groups=[],
+                       logit_rows=none, cu_q_host=cu, ctx_len_host=c["lens"], max_q_len=17, max_ctx_len=333,
+                       dtype=torch.bfloat16)
+    out = attention_mfma.try_attention(c["q"], c["kc"], c["vc"], c["table"], step, nq, window, c["scale"])
+    assert out is not None
+    err = (out.float().cpu() - c["want"]).abs().max()
+    assert torch.allclose(out.float().cpu(), c["want"], atol=1.5e-2, rtol=2e-2), err
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
