@@ -17,9 +17,9 @@
 // 8g .. 8g+7.  Keys are stored [page][kv head][slot][HD] and values transposed,
 // [page][kv head][HD][slot], so both A operands are plain 16-byte loads from the pages.
 //
-// With SPLIT, a tile's keys are divided among `nsplit` waves; each writes its unnormalised sums
-// and statistics to a scratch buffer and a second kernel merges them (decode with long contexts
-// and few requests).
+// Two kernels use this walk.  With many tiles (prompt portions) every wave owns a tile.  With
+// few tiles (decode) the waves of a block share one tile and merge through LDS; for very long
+// contexts the keys are further split among blocks, whose partial sums a second kernel merges.
 #include "common.h"
 
 #ifndef HD
@@ -57,10 +57,10 @@ struct TileState {
 __device__ __forceinline__ void attend(const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
                                        const int* __restrict__ bt, int table_width, int nkv, int kvh, int ps,
                                        const bf16x8_t* qb, int my_lo, int my_p, float scale_log2, int key_begin,
-                                       int key_end, TileState& st) {
+                                       int key_end, int kb_offset, int kb_stride, TileState& st) {
   const int lane = threadIdx.x & 63, lg = lane >> 4, r = lane & 15;
   const int max_key = table_width * ps - 1;
-  for (int kb = key_begin >> 5; (kb << 5) <= key_end; ++kb) {
+  for (int kb = (key_begin >> 5) + kb_offset; (kb << 5) <= key_end; kb += kb_stride) {
     const int key0 = kb << 5;
     // ---- S^T = K . Q^T for two blocks of 16 rows; row r of block b holds key 8*(r/4) + 4b + r%4
     f32x4_t s[2];
@@ -189,7 +189,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const bf16_t* __restrict
 #pragma unroll
   for (int dt = 0; dt < NT; ++dt) st.acc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   attend(kc, vc, bt + (size_t)r * table_width, table_width, nkv, kvh, ps, qb, t.my_lo, t.my_p, scale * LOG2E,
-         t.lo_tile, t.hi_tile, st);
+         t.lo_tile, t.hi_tile, 0, 1, st);
   if (!t.valid) return;
   const int lg = (threadIdx.x & 63) >> 4;
   const float inv = 1.0f / st.l;
@@ -204,27 +204,39 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const bf16_t* __restrict
   }
 }
 
-// ---- split over keys: partial sums to scratch, then a merge ---------------------------------
+// ---- few tiles (decode): the waves of a block share one tile ---------------------------------
+// The COOP_WAVES waves of a block take the tile's 32-key blocks in turn (wave w the blocks
+// w, w + COOP_WAVES, ...), then merge their sums and statistics through LDS in wave order.  With
+// nsplit > 1 the key range is further cut among blocks (grid.z); each block then writes its
+// merged partial to scratch and a second kernel merges the splits.
 // scratch layout per (tile, kv head, split): 16 columns x PART_COLS floats (HD sums, m, l, and
 // padding that keeps every column 16-byte aligned).
 #define PART_COLS (HD + 4)
 #define PART_STRIDE (16 * PART_COLS)
+#if HD <= 128
+#define COOP_WAVES 4
+#else
+#define COOP_WAVES 2
+#endif
 
-__global__ __launch_bounds__(256) void attn_mfma_split_kernel(
+__global__ __launch_bounds__(64 * COOP_WAVES) void attn_mfma_coop_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
     const int* __restrict__ bt, int table_width, const int* __restrict__ cu_q, const int* __restrict__ ctx_len,
-    const int* __restrict__ tile_req, const int* __restrict__ tile_ct, int num_tiles, float* __restrict__ scratch,
-    int nq, int nkv, int ps, int window, float scale, int nsplit, int keys_per_split) {
-  const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (item >= num_tiles * nsplit) return;
-  const int tile = item / nsplit, split = item - tile * nsplit;
-  const int kvh = blockIdx.y, g = nq / nkv;
+    const int* __restrict__ tile_req, const int* __restrict__ tile_ct, bf16_t* __restrict__ out,
+    float* __restrict__ scratch, int nq, int nkv, int ps, int window, float scale, int nsplit, int keys_per_split) {
+  __shared__ __attribute__((aligned(16))) float sm[COOP_WAVES][PART_STRIDE];
+  const int tile = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lg = lane >> 4, c = lane & 15;
+  const int g = nq / nkv;
   const int r = tile_req[tile], ct = tile_ct[tile];
   const TileInfo t = tile_info(cu_q, ctx_len, r, ct, g, kvh, window);
-  // splits are cut by absolute key index, in multiples of 32
-  const int first = (t.lo_tile >> 5 << 5) + split * keys_per_split;
-  int last = first + keys_per_split - 1;
-  last = last < t.hi_tile ? last : t.hi_tile;
+  int first = t.lo_tile, last = t.hi_tile;
+  if (nsplit > 1) {  // splits are cut by absolute key index, in multiples of 32
+    first = (t.lo_tile >> 5 << 5) + split * keys_per_split;
+    last = first + keys_per_split - 1;
+    last = last < t.hi_tile ? last : t.hi_tile;
+    first = first > t.lo_tile ? first : t.lo_tile;
+  }
   TileState st;
   st.m = -INFINITY;
   st.l = 0.f;
@@ -234,44 +246,84 @@ __global__ __launch_bounds__(256) void attn_mfma_split_kernel(
     bf16x8_t qb[KS];
     load_q(q, nq, t, qb);
     attend(kc, vc, bt + (size_t)r * table_width, table_width, nkv, kvh, ps, qb, t.my_lo, t.my_p, scale * LOG2E,
-           first, last, st);
+           first, last, wave, COOP_WAVES, st);
   }
-  const int lane = threadIdx.x & 63, lg = lane >> 4, c = lane & 15;
-  float* part = scratch + (((size_t)tile * nkv + kvh) * nsplit + split) * PART_STRIDE + (size_t)c * PART_COLS;
+  // every wave leaves its column sums in LDS: column c, channels dt*16 + 4*lg .. +3, then m and l
+  float* mine = &sm[wave][c * PART_COLS];
 #pragma unroll
-  for (int dt = 0; dt < NT; ++dt) {
-    const int d = dt * 16 + 4 * lg;
-    *reinterpret_cast<float4*>(part + d) = float4{st.acc[dt][0], st.acc[dt][1], st.acc[dt][2], st.acc[dt][3]};
-  }
+  for (int dt = 0; dt < NT; ++dt)
+    *reinterpret_cast<float4*>(mine + dt * 16 + 4 * lg) =
+        float4{st.acc[dt][0], st.acc[dt][1], st.acc[dt][2], st.acc[dt][3]};
   if (lg == 0) {
-    part[HD] = st.m;
-    part[HD + 1] = st.l;
+    mine[HD] = st.m;
+    mine[HD + 1] = st.l;
+  }
+  __syncthreads();
+  // merge: thread -> (column, 4 channels); waves are summed in order 0, 1, ...
+  for (int idx = threadIdx.x; idx < 16 * (HD / 4); idx += blockDim.x) {
+    const int col = idx / (HD / 4), d = (idx - col * (HD / 4)) * 4;
+    float m = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < COOP_WAVES; ++w) m = fmaxf(m, sm[w][col * PART_COLS + HD]);
+    float4 num = {0.f, 0.f, 0.f, 0.f};
+    float den = 0.f;
+#pragma unroll
+    for (int w = 0; w < COOP_WAVES; ++w) {
+      const float* p = &sm[w][col * PART_COLS];
+      const float wgt = (p[HD] == -INFINITY) ? 0.f : exp2f(p[HD] - m);
+      const float4 a = *reinterpret_cast<const float4*>(p + d);
+      num.x += wgt * a.x; num.y += wgt * a.y; num.z += wgt * a.z; num.w += wgt * a.w;
+      den += wgt * p[HD + 1];
+    }
+    const int colg = ct * 16 + col;
+    const int i = colg / g, gh = colg - i * g;
+    const int q0 = cu_q[r], qlen = cu_q[r + 1] - q0;
+    if (nsplit > 1) {
+      float* part = scratch + (((size_t)tile * nkv + kvh) * nsplit + split) * PART_STRIDE + (size_t)col * PART_COLS;
+      *reinterpret_cast<float4*>(part + d) = num;
+      if (d == 0) {
+        part[HD] = m;
+        part[HD + 1] = den;
+      }
+    } else if (i < qlen) {
+      const float inv = 1.0f / den;
+      uint2 wv;
+      wv.x = pack2(num.x * inv, num.y * inv);
+      wv.y = pack2(num.z * inv, num.w * inv);
+      *reinterpret_cast<uint2*>(out + ((size_t)(q0 + i) * nq + kvh * g + gh) * HD + d) = wv;
+    }
   }
 }
 
 __global__ void attn_mfma_merge_kernel(const float* __restrict__ scratch, const int* __restrict__ cu_q,
                                        const int* __restrict__ tile_req, const int* __restrict__ tile_ct,
                                        bf16_t* __restrict__ out, int nq, int nkv, int nsplit) {
-  // one block per (tile, kv head); thread = (column, channel group)
+  // one block per (tile, kv head); thread -> (column, 4 channels); splits are summed in order
   const int tile = blockIdx.x, kvh = blockIdx.y, g = nq / nkv;
   const int r = tile_req[tile], ct = tile_ct[tile];
   const int q0 = cu_q[r], qlen = cu_q[r + 1] - q0;
   const float* base = scratch + ((size_t)tile * nkv + kvh) * nsplit * PART_STRIDE;
-  for (int idx = threadIdx.x; idx < 16 * HD; idx += blockDim.x) {
-    const int c = idx / HD, d = idx - c * HD;
-    const int col = ct * 16 + c;
-    const int i = col / g, gh = col - i * g;
+  for (int idx = threadIdx.x; idx < 16 * (HD / 4); idx += blockDim.x) {
+    const int col = idx / (HD / 4), d = (idx - col * (HD / 4)) * 4;
+    const int colg = ct * 16 + col;
+    const int i = colg / g, gh = colg - i * g;
     if (i >= qlen) continue;
     float m = -INFINITY;
-    for (int s = 0; s < nsplit; ++s) m = fmaxf(m, base[(size_t)s * PART_STRIDE + c * PART_COLS + HD]);
-    float num = 0.f, den = 0.f;
+    for (int s = 0; s < nsplit; ++s) m = fmaxf(m, base[(size_t)s * PART_STRIDE + col * PART_COLS + HD]);
+    float4 num = {0.f, 0.f, 0.f, 0.f};
+    float den = 0.f;
     for (int s = 0; s < nsplit; ++s) {
-      const float* p = base + (size_t)s * PART_STRIDE + c * PART_COLS;
-      const float w = (p[HD] == -INFINITY) ? 0.f : exp2f(p[HD] - m);
-      num += w * p[d];
-      den += w * p[HD + 1];
+      const float* p = base + (size_t)s * PART_STRIDE + col * PART_COLS;
+      const float wgt = (p[HD] == -INFINITY) ? 0.f : exp2f(p[HD] - m);
+      const float4 a = *reinterpret_cast<const float4*>(p + d);
+      num.x += wgt * a.x; num.y += wgt * a.y; num.z += wgt * a.z; num.w += wgt * a.w;
+      den += wgt * p[HD + 1];
     }
-    out[((size_t)(q0 + i) * nq + kvh * g + gh) * HD + d] = f32_to_bf16(num / den);
+    const float inv = 1.0f / den;
+    uint2 wv;
+    wv.x = pack2(num.x * inv, num.y * inv);
+    wv.y = pack2(num.z * inv, num.w * inv);
+    *reinterpret_cast<uint2*>(out + ((size_t)(q0 + i) * nq + kvh * g + gh) * HD + d) = wv;
   }
 }
 
@@ -302,20 +354,21 @@ extern "C" long long qvl_attn_mfma_scratch_floats(int num_tiles, int nkv, int ns
   return (long long)num_tiles * nkv * nsplit * PART_STRIDE;
 }
 
-extern "C" int qvl_attn_mfma_split(const void* q, const void* kc, const void* vc, const void* bt, int table_width,
-                                   const void* cu_q, const void* ctx_len, const void* tile_req, const void* tile_ct,
-                                   int num_tiles, void* out, void* scratch, int nq, int nkv, int ps, int window,
-                                   float scale, int nsplit, int keys_per_split, hipStream_t stream) {
+extern "C" int qvl_attn_mfma_coop(const void* q, const void* kc, const void* vc, const void* bt, int table_width,
+                                  const void* cu_q, const void* ctx_len, const void* tile_req, const void* tile_ct,
+                                  int num_tiles, void* out, void* scratch, int nq, int nkv, int ps, int window,
+                                  float scale, int nsplit, int keys_per_split, hipStream_t stream) {
   const int c = check_common(num_tiles, nq, nkv, ps, table_width);
   if (c >= 0) return c;
-  if (nsplit <= 0 || keys_per_split <= 0 || keys_per_split % 32) return QVL_ERR_SHAPE;
-  const dim3 grid((num_tiles * nsplit + 3) / 4, nkv);
-  hipLaunchKernelGGL(attn_mfma_split_kernel, grid, dim3(256), 0, stream, (const bf16_t*)q, (const bf16_t*)kc,
-                     (const bf16_t*)vc, (const int*)bt, table_width, (const int*)cu_q, (const int*)ctx_len,
-                     (const int*)tile_req, (const int*)tile_ct, num_tiles, (float*)scratch, nq, nkv, ps, window,
-                     scale, nsplit, keys_per_split);
+  if (nsplit <= 0 || nsplit > 65535 || (nsplit > 1 && (keys_per_split <= 0 || keys_per_split % 32 || !scratch)))
+    return QVL_ERR_SHAPE;
+  hipLaunchKernelGGL(attn_mfma_coop_kernel, dim3(num_tiles, nkv, nsplit), dim3(64 * COOP_WAVES), 0, stream,
+                     (const bf16_t*)q, (const bf16_t*)kc, (const bf16_t*)vc, (const int*)bt, table_width,
+                     (const int*)cu_q, (const int*)ctx_len, (const int*)tile_req, (const int*)tile_ct, (bf16_t*)out,
+                     (float*)scratch, nq, nkv, ps, window, scale, nsplit, keys_per_split);
   if (hipGetLastError() != hipSuccess) return QVL_ERR_LAUNCH;
-  hipLaunchKernelGGL(attn_mfma_merge_kernel, dim3(num_tiles, nkv), dim3(256), 0, stream, (const float*)scratch,
-                     (const int*)cu_q, (const int*)tile_req, (const int*)tile_ct, (bf16_t*)out, nq, nkv, nsplit);
+  if (nsplit > 1)
+    hipLaunchKernelGGL(attn_mfma_merge_kernel, dim3(num_tiles, nkv), dim3(256), 0, stream, (const float*)scratch,
+                       (const int*)cu_q, (const int*)tile_req, (const int*)tile_ct, (bf16_t*)out, nq, nkv, nsplit);
   return qvl_launch_status();
 }

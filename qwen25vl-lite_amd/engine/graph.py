@@ -1,0 +1,156 @@
+"""Decode steps replayed from HIP graphs.
+
+A decode step of a 7B model is a few hundred short kernels; launched one by one from Python
+the host, not the GPU, sets the step time (the reference measured the same on its hardware,
+reference src/qwen25vl_lite/graphs.py:3-7, and also answers with graph capture).  A step in
+which every request brings exactly one token has a fixed shape, so it is captured once per
+(batch size, context bucket) and replayed: per step the host fills one pinned buffer with the
+step's integers (token ids, positions, page slots, block tables, context lengths), copies it to
+a fixed device buffer in one transfer, and launches the graph.
+
+The context bucket (the next power of two above the longest context) only fixes how many waves
+the attention kernel splits a request's keys over; the true lengths travel in the buffer.
+"""
+
+from __future__ import annotations
+
+from typing import Dict, List, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from ..parts.base import GroupStep, StepContext
+from .batch import StepEntry
+
+__all__ = ["DecodeGraphs"]
+
+
+def _bucket(n: int, floor: int = 256) -> int:
+    b = floor
+    while b < n:
+        b *= 2
+    return b
+
+
+class _Graph:
+    """One captured step shape: its buffers, its StepContext of fixed views, its graph."""
+
+    def __init__(self, runner, batch: int, ctx_bucket: int):
+        self.runner = runner
+        self.batch = batch
+        cache = runner.cache
+        self.ngroups = len(cache.groups)
+        self.rows = runner.model.spec.position_rows
+        self.width = runner.ecfg.max_blocks_per_seq
+        self.ps = cache.page_size
+        b, w = batch, self.width
+        sizes = [("token_ids", b), ("positions", self.rows * b), ("token_req", b), ("token_seqpos", b),
+                 ("cu_q", b + 1), ("ctx_len", b), ("req_slots", b), ("logit_rows", b)]
+        for g in range(self.ngroups):
+            sizes += [(f"slots{g}", b), (f"table{g}", b * w)]
+        self.offsets: Dict[str, Tuple[int, int]] = {}
+        total = 0
+        for name, n in sizes:
+            self.offsets[name] = (total, n)
+            total += (n + 3) // 4 * 4
+        self.host = torch.zeros(total, dtype=torch.int32, pin_memory=True)
+        self.hv = self.host.numpy()
+        self.dev = torch.zeros(total, dtype=torch.int32, device=runner.device)
+        self.copied = torch.cuda.Event()
+        self.copied.record()
+
+        def h(name, shape=None):
+            o, n = self.offsets[name]
+            v = self.hv[o:o + n]
+            return v if shape is None else v.reshape(shape)
+
+        def d(name, shape=None):
+            o, n = self.offsets[name]
+            v = self.dev[o:o + n]
+            return v if shape is None else v.view(shape)
+
+        self.h = h
+        h("token_req")[:] = np.arange(b)
+        h("cu_q")[:] = np.arange(b + 1)
+        h("logit_rows")[:] = np.arange(b)
+        for g in range(self.ngroups):
+            h(f"table{g}")[:] = -1
+        self.tables = [h(f"table{g}", (b, w)) for g in range(self.ngroups)]
+        self.row_req: List[object] = [None] * b
+        self.row_len = [[0] * b for _ in range(self.ngroups)]
+        self.step = StepContext(
+            num_tokens=b, num_reqs=b, token_ids=d("token_ids"), positions=d("positions", (self.rows, b)),
+            token_req=d("token_req"), token_seqpos=d("token_seqpos"), cu_q=d("cu_q"), ctx_len=d("ctx_len"),
+            req_slots=d("req_slots"),
+            groups=[GroupStep(d(f"slots{g}"), d(f"table{g}", (b, w)), self.ps) for g in range(self.ngroups)],
+            logit_rows=d("logit_rows"), cu_q_host=list(range(b + 1)), ctx_len_host=[ctx_bucket] * b,
+            req_slots_host=[0] * b, max_q_len=1, max_ctx_len=ctx_bucket, dtype=runner.dtype)
+        self.graph = None
+        self.logits = None
+
+    def fill(self, entries: Sequence[StepEntry]) -> None:
+        cache, ps, h = self.runner.cache, self.ps, self.h
+        self.copied.synchronize()          # the previous transfer has read the pinned buffer
+        starts = np.fromiter((e.start for e in entries), np.int32, self.batch)
+        deltas = np.fromiter((e.rope_delta for e in entries), np.int32, self.batch)
+        h("token_ids")[:] = np.fromiter((e.tokens[0] for e in entries), np.int32, self.batch)
+        h("token_seqpos")[:] = starts
+        h("positions", (self.rows, self.batch))[:] = starts + deltas
+        h("ctx_len")[:] = starts + 1
+        h("req_slots")[:] = np.fromiter((cache.slot_of(e.req_id) for e in entries), np.int32, self.batch)
+        for g in range(self.ngroups):
+            table_np, lens, slots = self.tables[g], self.row_len[g], h(f"slots{g}")
+            for i, e in enumerate(entries):
+                t = cache.table(e.req_id, g)
+                if self.row_req[i] is not cache.requests[e.req_id]:   # another request, or this one admitted anew
+                    table_np[i, :] = -1
+                    lens[i] = 0
+                if len(t) > lens[i]:
+                    # pages only ever join at the end; entries a window has given back are never read
+                    table_np[i, lens[i]:len(t)] = t[lens[i]:]
+                    lens[i] = len(t)
+                slots[i] = t[e.start // ps] * ps + e.start % ps
+        for i, e in enumerate(entries):
+            self.row_req[i] = cache.requests[e.req_id]
+
+    def run(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        runner = self.runner
+        self.fill(entries)
+        self.dev.copy_(self.host, non_blocking=True)
+        self.copied.record()
+        if self.graph is None:
+            # twice eagerly (libraries pick kernels and workspaces, per-step tile lists are made),
+            # then once more under capture; a decode step only writes the step's own cache slots
+            # and the logits, so running it again with the same inputs changes nothing
+            for _ in range(2):
+                runner.model.forward(self.step, runner.slots)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                self.logits = runner.model.forward(self.step, runner.slots)
+            self.graph = graph
+        self.graph.replay()
+        return self.logits
+
+
+class DecodeGraphs:
+    """The graphs of a runner, keyed by (batch size, context bucket)."""
+
+    def __init__(self, runner, max_graphs: int = 32):
+        self.runner = runner
+        self.max_graphs = max_graphs
+        self.graphs: Dict[Tuple[int, int], _Graph] = {}
+
+    @staticmethod
+    def takes(entries: Sequence[StepEntry]) -> bool:
+        return all(len(e.tokens) == 1 and e.positions is None and list(e.want) == [0] for e in entries)
+
+    def run(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        ctx = max(e.start for e in entries) + 1
+        key = (len(entries), _bucket(ctx))
+        g = self.graphs.get(key)
+        if g is None:
+            if len(self.graphs) >= self.max_graphs:
+                self.graphs.pop(next(iter(self.graphs)))
+            g = self.graphs[key] = _Graph(self.runner, *key)
+        return g.run(entries)

@@ -46,7 +46,13 @@ class ModelRunner:
             for need in model.entry_state
         ]
         self.slots = model.make_slots(self.storage, self.states)
+        self.position_rows = model.spec.position_rows
         self.steps = 0
+        # decode steps from HIP graphs, if asked for and every part can be captured
+        self.graphs = None
+        if engine_cfg.hip_graph and model.graph_safe:
+            from .graph import DecodeGraphs
+            self.graphs = DecodeGraphs(self)
 
     # ------------------------------------------------------------------ requests
     def admit(self, req_id) -> int:
@@ -73,9 +79,16 @@ class ModelRunner:
             self.cache.reserve(e.req_id, e.start + len(e.tokens))
         self._clear_state(entries)
         with torch.cuda.device(self.device):
-            step = build_step(entries, self.cache, self.model.spec.position_rows, self.dtype, self.device,
-                              self.vocab_size)
-            logits = self.model.forward(step, self.slots)
+            if self.graphs is not None and self.graphs.takes(entries):
+                for e in entries:
+                    if not 0 <= e.tokens[0] < self.vocab_size:
+                        raise ValueError(f"request {e.req_id!r}: token id outside [0, {self.vocab_size})")
+                    if self.cache.num_tokens(e.req_id) != e.start:
+                        raise ValueError(f"request {e.req_id!r}: the step does not continue where the cache ends")
+                logits = self.graphs.run(entries)
+            else:
+                step = build_step(entries, self.cache, self.position_rows, self.dtype, self.device, self.vocab_size)
+                logits = self.model.forward(step, self.slots)
         for e in entries:
             self.cache.commit(e.req_id, e.start + len(e.tokens))
         self.steps += 1

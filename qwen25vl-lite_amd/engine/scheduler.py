@@ -250,7 +250,11 @@ class LLMEngine:
 
     def _entry(self, seq: Sequence_, n: int) -> StepEntry:
         start = seq.num_computed_tokens
-        tokens = seq.tokens[start:start + n]
+        p_len = len(seq.prompt_token_ids)
+        if start >= p_len:
+            tokens = seq.output_token_ids[start - p_len:start - p_len + n]
+        else:
+            tokens = seq.tokens[start:start + n]
         positions = None
         if seq.prompt_positions is not None and start < len(seq.prompt_token_ids):
             p_len = len(seq.prompt_token_ids)

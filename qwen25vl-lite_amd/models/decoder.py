@@ -91,6 +91,13 @@ class DecoderModel:
         self.params[spec.head_name] = (None, "head", ParamSpec((spec.vocab_size, spec.hidden_size), "matrix"))
 
     # ------------------------------------------------------------------ structure
+    @property
+    def graph_safe(self) -> bool:
+        """True if every part may run under HIP graph capture."""
+        def safe(part) -> bool:
+            return part.graph_safe and all(safe(s) for s in part.sub_parts().values())
+        return all(safe(b) for b in self.blocks) and safe(self.final_norm)
+
     def cache_groups(self) -> List[CacheGroupSpec]:
         return [CacheGroupSpec(need, n) for need, n in zip(self.group_needs, self.group_layers)]
 

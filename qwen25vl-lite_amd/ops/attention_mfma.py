@@ -19,8 +19,9 @@ __all__ = ["try_attention", "supports", "tiles_for", "plan_splits"]
 
 _c_int, _c_float, _c_ptr = ctypes.c_int, ctypes.c_float, ctypes.c_void_p
 _MAX_HD = 256
-TARGET_WAVES = 1024      # enough waves to fill 256 compute units
-MIN_KEYS_PER_SPLIT = 64
+TARGET_BLOCKS = 512        # from here on a wave per tile fills the 256 compute units
+FILL_BLOCKS = 256          # with fewer cooperative blocks than this, long contexts are split
+MIN_KEYS_PER_SPLIT = 1024  # a split is worth a second kernel only above this many keys
 
 
 def supports(head_dim: int, dtype: torch.dtype) -> bool:
@@ -37,15 +38,19 @@ def tiles_for(cu_q, group: int) -> Tuple[np.ndarray, np.ndarray]:
     return req, ct
 
 
-def plan_splits(num_tiles: int, nkv: int, max_ctx: int) -> Tuple[int, int]:
-    """``(nsplit, keys_per_split)``; nsplit 1 means the unsplit kernel."""
-    waves = num_tiles * nkv
-    if waves >= TARGET_WAVES // 2 or max_ctx <= 2 * MIN_KEYS_PER_SPLIT:
-        return 1, 0
-    want = (TARGET_WAVES + waves - 1) // waves
-    per = max(MIN_KEYS_PER_SPLIT, ((max_ctx + want - 1) // want + 31) // 32 * 32)
-    nsplit = (max_ctx + 31 + per - 1) // per
-    return (nsplit, per) if nsplit > 1 else (1, 0)
+def plan_splits(num_tiles: int, nkv: int, max_ctx: int) -> Tuple[str, int, int]:
+    """``(kernel, nsplit, keys_per_split)``.  ``"tile"``: every wave owns a tile (many tiles, as in
+    prefill).  ``"coop"``: the waves of a block share a tile (few tiles, as in decode); its keys are
+    split among ``nsplit`` blocks when the context is long and the blocks are few."""
+    blocks = num_tiles * nkv
+    if blocks >= TARGET_BLOCKS:
+        return "tile", 1, 0
+    want = (FILL_BLOCKS + blocks - 1) // blocks
+    nsplit = max(1, min(want, max_ctx // MIN_KEYS_PER_SPLIT))
+    if nsplit == 1:
+        return "coop", 1, 0
+    per = ((max_ctx + 31 + nsplit - 1) // nsplit + 31) // 32 * 32
+    return "coop", (max_ctx + 31 + per - 1) // per, per
 
 
 def _step_tiles(step, group: int, device):
@@ -74,18 +79,20 @@ def try_attention(q, k_cache, v_cache, block_table, step, num_q_heads: int, wind
     tile_req, tile_ct, num_tiles = _step_tiles(step, nq // nkv, q.device)
     out = torch.empty_like(q)
     defines = {"HD": hd}
-    nsplit, per = plan_splits(num_tiles, nkv, step.max_ctx_len)
+    kind, nsplit, per = plan_splits(num_tiles, nkv, step.max_ctx_len)
     common = [_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(step.cu_q),
               _ptr(step.ctx_len), _ptr(tile_req), _ptr(tile_ct), num_tiles, _ptr(out)]
-    if nsplit == 1:
+    if kind == "tile":
         fn = _fn("attention_mfma", "qvl_attn_mfma",
                  [_c_ptr] * 4 + [_c_int] + [_c_ptr] * 4 + [_c_int, _c_ptr] + [_c_int] * 4 + [_c_float, _c_ptr], defines)
         _check(fn(*common, nq, nkv, ps, int(window or 0), float(scale), _stream()), "paged_attention (matrix cores)")
     else:
-        scratch = torch.empty(num_tiles * nkv * nsplit * 16 * (hd + 4), dtype=torch.float32, device=q.device)
-        fn = _fn("attention_mfma", "qvl_attn_mfma_split",
+        scratch = None
+        if nsplit > 1:
+            scratch = torch.empty(num_tiles * nkv * nsplit * 16 * (hd + 4), dtype=torch.float32, device=q.device)
+        fn = _fn("attention_mfma", "qvl_attn_mfma_coop",
                  [_c_ptr] * 4 + [_c_int] + [_c_ptr] * 4 + [_c_int, _c_ptr, _c_ptr] + [_c_int] * 4
                  + [_c_float, _c_int, _c_int, _c_ptr], defines)
         _check(fn(*common, _ptr(scratch), nq, nkv, ps, int(window or 0), float(scale), nsplit, per, _stream()),
-               "paged_attention (matrix cores, split)")
+               "paged_attention (matrix cores, shared tiles)")
     return out

@@ -26,6 +26,8 @@ class PagedAttention(Mixer):
     ``position`` (a :class:`PartSpec` of category ``position``), ``kv_shared`` (True: the layer
     has no key/value projections and reads the cache another layer wrote)."""
 
+    graph_safe = True
+
     def __init__(self, params, dtype, device):
         super().__init__(dtype, device)
         self.hidden = int(params["hidden_size"])

@@ -125,7 +125,11 @@ class ResidualStream:
 
 
 class Part:
-    """Base of all parts."""
+    """Base of all parts.  ``graph_safe`` says that ``forward`` only launches device work whose
+    shape depends on the step's shape alone (no host reads of device data, no host loops over
+    the step's values), so a decode step through it may be captured in a HIP graph."""
+
+    graph_safe: bool = False
 
     def __init__(self, dtype: torch.dtype, device: torch.device):
         self.dtype = dtype

@@ -17,6 +17,8 @@ class PreNormBlock(Block):
     inside the following norm's kernel (the last one in the model's final norm).
     """
 
+    graph_safe = True
+
     def __init__(self, params, dtype, device):
         super().__init__(dtype, device)
         self.norm1 = build_part("norm", params["norm1"], dtype, device)

@@ -19,6 +19,8 @@ class SwiGLU(FeedForward):
     params: ``hidden_size``, ``intermediate_size``.
     """
 
+    graph_safe = True
+
     def __init__(self, params, dtype, device):
         super().__init__(dtype, device)
         self.hidden = int(params["hidden_size"])

@@ -19,6 +19,8 @@ class RMSNorm(Norm):
     params: ``size`` (row width), ``eps``.
     """
 
+    graph_safe = True
+
     def __init__(self, params, dtype, device):
         super().__init__(dtype, device)
         self.size = int(params["size"])

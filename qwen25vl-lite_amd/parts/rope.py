@@ -33,6 +33,8 @@ class MRoPE(PositionEncoding):
 
     num_rows = 3
 
+    graph_safe = True
+
     def __init__(self, params, dtype, device):
         super().__init__(dtype, device)
         self.theta = float(params["theta"])
@@ -61,6 +63,8 @@ class RoPE1D(PositionEncoding):
     """params: ``theta``, optional ``rotary_dim`` (default: the whole head)."""
 
     num_rows = 1
+
+    graph_safe = True
 
     def __init__(self, params, dtype, device):
         super().__init__(dtype, device)

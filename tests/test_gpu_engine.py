@@ -59,6 +59,30 @@ def test_long_decode_and_preemption(model_dirs):
     assert llm.runner.cache.pages_in_use() == [0, 0]
 
 
+@pytest.mark.parametrize("name, dtype", [("B_sharp", "float32"), ("C_sharp", "bfloat16"), ("A", "bfloat16")])
+def test_decode_from_hip_graphs_gives_the_same_tokens(model_dirs, name, dtype):
+    """Decode steps replayed from HIP graphs, many replays with eager prefill steps, admissions and
+    finishes in between (batch size and context bucket change): every token equals the eager run's."""
+    from qwen25vl_lite_amd import LLM, SamplingParams
+
+    d = model_dirs[name]
+    vocab = {"A": 256, "B": 509, "C": 300}[name[0]]
+    prompts = [random_tokens(n, vocab, 50 + n) for n in (5, 250, 31, 70, 12)]
+    params = [SamplingParams(temperature=0.0, max_tokens=m, ignore_eos=True) for m in (40, 30, 60, 9, 25)]
+    common = dict(dtype=dtype, num_blocks=64, block_size=16, max_num_seqs=3, max_num_batched_tokens=64,
+                  enable_prefix_cache=False)
+    eager = LLM(d, **common).generate(prompts, params)
+    llm = LLM(d, hip_graph=True, **common)
+    assert llm.runner.graphs is not None
+    graphed = llm.generate(prompts, params)
+    assert len(llm.runner.graphs.graphs) >= 3
+    for a, b in zip(eager, graphed):
+        assert a.output_token_ids == b.output_token_ids
+    if dtype == "float32":
+        for prompt, out, p in zip(prompts, graphed, params):
+            assert out.output_token_ids == _plain_greedy(d, prompt, p.max_tokens)
+
+
 def test_prefix_reuse_gives_the_same_tokens(model_dirs):
     # reference tests/test_chunked_prefill.py:193-227, tests/test_engine.py:57-106
     from qwen25vl_lite_amd import LLM, SamplingParams

@@ -162,14 +162,16 @@ def test_paged_attention_generic(dtype, nq, nkv, hd, window):
     assert torch.allclose(out.float().cpu(), c["want"], **tol), (out.float().cpu() - c["want"]).abs().max()
 
 
-@pytest.mark.parametrize("split", [False, True])
+@pytest.mark.parametrize("split", ["tile", "coop", "coop_split"])
 @pytest.mark.parametrize("nq, nkv, hd, window", [s for s in ATTN_SHAPES if s[2] % 16 == 0])
 def test_paged_attention_matrix_cores(nq, nkv, hd, window, split, monkeypatch):
-    """The matrix-core kernel on the same case, unsplit and with the keys split among waves."""
+    """The matrix-core kernels on the same case: a wave per tile, the waves of a block sharing a
+    tile, and the keys further split among blocks."""
     from qwen25vl_lite_amd.ops import attention_mfma
     from qwen25vl_lite_amd.parts import StepContext
     c = _attention_case(torch.bfloat16, nq, nkv, hd, window)
-    monkeypatch.setattr(attention_mfma, "plan_splits", (lambda t, n, m: (7, 64)) if split else (lambda t, n, m: (1, 0)))
+    plan = {"tile": ("tile", 1, 0), "coop": ("coop", 1, 0), "coop_split": ("coop", 6, 64)}[split]
+    monkeypatch.setattr(attention_mfma, "plan_splits", lambda t, n, m: plan)
     cu = [0]
     for ql in c["qlens"]:
         cu.append(cu[-1] + ql)
@@ -212,16 +214,29 @@ def test_gemm_f32_is_exact_and_row_independent(m, n, k):
     assert torch.equal(alone[0], out[m // 2])
 
 
-@pytest.mark.parametrize("m, n, k", [(1, 509, 144), (8, 300, 200), (33, 130, 352), (300, 64, 1000)])
+@pytest.mark.parametrize("m, n, k", [(1, 509, 144), (8, 300, 200), (16, 17, 8), (17, 1000, 4104), (31, 130, 352),
+                                     (64, 509, 3584), (5, 40, 100), (300, 64, 1000)])
 def test_linear_bfloat16(m, n, k):
+    """Few rows go through the skinny matrix-core kernel (inner sizes in steps of 8), the rest
+    through the library; both accumulate in float32."""
+    from qwen25vl_lite_amd.ops import skinny
     from qwen25vl_lite_amd.ops.linear import linear
     torch.manual_seed(k)
     x, w = torch.randn(m, k).bfloat16(), (torch.randn(n, k) / math.sqrt(k)).bfloat16()
+    b = torch.randn(n)
     want = x.float() @ w.float().T
+    took = skinny.try_linear(x.cuda(), w.cuda(), None, torch.float32)
+    assert (took is not None) == (m <= 32 and k % 8 == 0)
     out32 = linear(x.cuda(), w.cuda(), out_dtype=torch.float32)
     assert out32.dtype == torch.float32 and torch.allclose(out32.cpu(), want, atol=2e-3, rtol=2e-3)
     out16 = linear(x.cuda(), w.cuda())
     assert out16.dtype == torch.bfloat16 and torch.allclose(out16.float().cpu(), want, atol=2e-2, rtol=2e-2)
+    outb = linear(x.cuda(), w.cuda(), b.cuda(), out_dtype=torch.float32)
+    assert torch.allclose(outb.cpu(), want + b, atol=2e-3, rtol=2e-3)
+    # a row's result does not depend on the rows beside it
+    if m > 1:
+        alone = linear(x[m // 2:m // 2 + 1].contiguous().cuda(), w.cuda(), out_dtype=torch.float32)
+        assert torch.allclose(alone[0], out32[m // 2], atol=1e-5, rtol=1e-5)
 
 
 def test_no_cpu_path():
