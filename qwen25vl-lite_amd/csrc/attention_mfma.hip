@@ -53,33 +53,65 @@ struct TileState {
   f32x4_t acc[NT];
 };
 
-// Walk keys [key_begin, key_end] (inclusive, absolute) of one tile.
-__device__ __forceinline__ void attend(const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
-                                       const int* __restrict__ bt, int table_width, int nkv, int kvh, int ps,
-                                       const bf16x8_t* qb, int my_lo, int my_p, float scale_log2, int key_begin,
-                                       int key_end, int kb_offset, int kb_stride, TileState& st) {
-  const int lane = threadIdx.x & 63, lg = lane >> 4, r = lane & 15;
-  const int max_key = table_width * ps - 1;
-  for (int kb = (key_begin >> 5) + kb_offset; (kb << 5) <= key_end; kb += kb_stride) {
-    const int key0 = kb << 5;
-    // ---- S^T = K . Q^T for two blocks of 16 rows; row r of block b holds key 8*(r/4) + 4b + r%4
-    f32x4_t s[2];
+// The page of each key row this lane loads in one 32-key block (two K row blocks, one V group).
+struct BlockPages {
+  int k[2], v;
+};
+// One 32-key block in registers: K rows as A operands of S^T, V^T rows as A operands of O^T.
+struct BlockRegs {
+  bf16x8_t k[2][KS];
+  bf16x8_t v[NT];
+};
+
+struct Walk {
+  const bf16_t* kc;
+  const bf16_t* vc;
+  const int* bt;  // this request's row of the block table
+  int max_key, nkv, kvh, ps;
+  int my_lo, my_p, key_begin, key_end;
+  float scale_log2;
+  int lg, r;
+
+  // Row r of K block b holds key 8*(r/4) + 4b + r%4, so that after the product lane group lg
+  // holds the 8 consecutive keys 8*lg .. 8*lg+7 (see the top of the file).
+  __device__ __forceinline__ int krow_key(int kb, int b) const { return (kb << 5) + 8 * (r >> 2) + 4 * b + (r & 3); }
+
+  __device__ __forceinline__ void issue_pages(int kb, BlockPages& pg) const {
+#pragma unroll
+    for (int b = 0; b < 2; ++b) pg.k[b] = bt[min(krow_key(kb, b), max_key) / ps];
+    pg.v = bt[min((kb << 5) + 8 * lg, max_key) / ps];
+  }
+
+  __device__ __forceinline__ void issue_loads(int kb, const BlockPages& pg, BlockRegs& rg) const {
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
-      const int key = key0 + 8 * (r >> 2) + 4 * b + (r & 3);
-      int page = bt[min(key, max_key) / ps];
-      page = page < 0 ? 0 : page;
+      const int key = krow_key(kb, b);
+      const int page = pg.k[b] < 0 ? 0 : pg.k[b];  // keys nobody sees may have no page: read page 0, masked later
       const bf16_t* krow = kc + (((size_t)page * nkv + kvh) * ps + (size_t)(key % ps)) * HD;
-      f32x4_t a = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         const int d = ks * 32 + 8 * lg;
-        const bf16x8_t kk = (d < HD) ? load8(krow + d) : zero8();
-        a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kk, qb[ks], a, 0, 0, 0);
+        rg.k[b][ks] = (d < HD) ? load8(krow + d) : zero8();
       }
+    }
+    const int vkey = (kb << 5) + 8 * lg;
+    const int vpage = (pg.v < 0 || vkey > max_key) ? 0 : pg.v;
+    const bf16_t* vbase = vc + (((size_t)vpage * nkv + kvh) * HD) * ps + (size_t)(vkey % ps);
+#pragma unroll
+    for (int dt = 0; dt < NT; ++dt) rg.v[dt] = load8(vbase + (size_t)(dt * 16 + r) * ps);
+  }
+
+  __device__ __forceinline__ void compute(int kb, const bf16x8_t* qb, const BlockRegs& rg, TileState& st) const {
+    const int key0 = kb << 5;
+    f32x4_t s[2];
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      f32x4_t a = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(rg.k[b][ks], qb[ks], a, 0, 0, 0);
       s[b] = a;
     }
-    // ---- mask and online softmax; this lane holds keys key0 + 8*lg + j of column r
+    // mask and online softmax; this lane holds keys key0 + 8*lg + j of column r
     float sv[8];
     float mloc = -INFINITY;
 #pragma unroll
@@ -112,19 +144,48 @@ __device__ __forceinline__ void attend(const bf16_t* __restrict__ kc, const bf16
     st.m = m_new;
     u32x4_t packed = {pack2(pv[0], pv[1]), pack2(pv[2], pv[3]), pack2(pv[4], pv[5]), pack2(pv[6], pv[7])};
     const bf16x8_t pb = __builtin_bit_cast(bf16x8_t, packed);
-    // ---- O^T += V^T . P^T; this lane reads keys key0 + 8*lg .. +7 of channel dt*16 + r
-    const int vkey = key0 + 8 * lg;
-    int vpage = bt[min(vkey, max_key) / ps];
-    vpage = (vpage < 0 || vkey > max_key) ? 0 : vpage;
-    const bf16_t* vbase = vc + (((size_t)vpage * nkv + kvh) * HD) * ps + (size_t)(vkey % ps);
 #pragma unroll
     for (int dt = 0; dt < NT; ++dt) {
-      const bf16x8_t vv = load8(vbase + (size_t)(dt * 16 + r) * ps);
       f32x4_t o = st.acc[dt];
       o[0] *= alpha; o[1] *= alpha; o[2] *= alpha; o[3] *= alpha;
-      st.acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv, pb, o, 0, 0, 0);
+      st.acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(rg.v[dt], pb, o, 0, 0, 0);
     }
   }
+};
+
+// Walk the 32-key blocks first, first + stride, ... that overlap keys [key_begin, key_end]
+// (inclusive, absolute) of one tile.  The loads of the next block and the page lookups of the one
+// after are issued before the current block is computed, so a wave always has a block in flight.
+__device__ __forceinline__ void attend(const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
+                                       const int* __restrict__ bt, int table_width, int nkv, int kvh, int ps,
+                                       const bf16x8_t* qb, int my_lo, int my_p, float scale_log2, int key_begin,
+                                       int key_end, int kb_offset, int kb_stride, TileState& st) {
+  const int lane = threadIdx.x & 63;
+  Walk w;
+  w.kc = kc; w.vc = vc; w.bt = bt;
+  w.max_key = table_width * ps - 1; w.nkv = nkv; w.kvh = kvh; w.ps = ps;
+  w.my_lo = my_lo; w.my_p = my_p; w.key_begin = key_begin; w.key_end = key_end;
+  w.scale_log2 = scale_log2; w.lg = lane >> 4; w.r = lane & 15;
+  const int s = kb_stride;
+  int kb = (key_begin >> 5) + kb_offset;
+#define LIVE(x) (((x) << 5) <= key_end)
+  if (!LIVE(kb)) return;
+  BlockPages p0, p1;
+  BlockRegs ra, rb;
+  w.issue_pages(kb, p0);
+  if (LIVE(kb + s)) w.issue_pages(kb + s, p1);
+  w.issue_loads(kb, p0, ra);
+  for (;; kb += 2 * s) {
+    if (LIVE(kb + 2 * s)) w.issue_pages(kb + 2 * s, p0);
+    if (LIVE(kb + s)) w.issue_loads(kb + s, p1, rb);
+    w.compute(kb, qb, ra, st);
+    if (!LIVE(kb + s)) break;
+    if (LIVE(kb + 3 * s)) w.issue_pages(kb + 3 * s, p1);
+    if (LIVE(kb + 2 * s)) w.issue_loads(kb + 2 * s, p0, ra);
+    w.compute(kb + s, qb, rb, st);
+    if (!LIVE(kb + 2 * s)) break;
+  }
+#undef LIVE
 }
 
 // Everything a wave needs to know about its tile.

@@ -65,15 +65,78 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__
   }
 }
 
+// The same with every value held in registers between the two passes: rows whose width is a
+// multiple of 4 and at most NORM_VEC_MAX * 4 * 256, read and written 4 values at a time.
+#define NORM_VEC_MAX 8
+
+template <typename T> __device__ __forceinline__ float4 ld4(const T* p);
+template <> __device__ __forceinline__ float4 ld4<float>(const float* p) { return *reinterpret_cast<const float4*>(p); }
+template <> __device__ __forceinline__ float4 ld4<bf16_t>(const bf16_t* p) {
+  const uint2 v = *reinterpret_cast<const uint2*>(p);
+  return float4{__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u), __uint_as_float(v.y << 16),
+                __uint_as_float(v.y & 0xffff0000u)};
+}
+template <typename T> __device__ __forceinline__ void st4(T* p, float4 v);
+template <> __device__ __forceinline__ void st4<float>(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+template <> __device__ __forceinline__ void st4<bf16_t>(bf16_t* p, float4 v) {
+  uint2 o;
+  o.x = (uint32_t)f32_to_bf16(v.x) | ((uint32_t)f32_to_bf16(v.y) << 16);
+  o.y = (uint32_t)f32_to_bf16(v.z) | ((uint32_t)f32_to_bf16(v.w) << 16);
+  *reinterpret_cast<uint2*>(p) = o;
+}
+
+template <typename TD, typename TO>
+__global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict__ h, const TD* __restrict__ delta,
+                                                              const float* __restrict__ w, TO* __restrict__ out,
+                                                              const int* __restrict__ rows, int H, float eps) {
+  __shared__ float red[17];
+  const int m = blockIdx.x;
+  const int row = rows ? rows[m] : m;
+  float* hr = h + (size_t)row * H;
+  const TD* dr = delta ? delta + (size_t)row * H : nullptr;
+  const int nvec = H >> 2;
+  float4 v[NORM_VEC_MAX];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < NORM_VEC_MAX; ++j) {
+    const int i = threadIdx.x + 256 * j;
+    if (i < nvec) {
+      float4 x = ld4<float>(hr + 4 * i);
+      if (dr) {
+        const float4 d = ld4<TD>(dr + 4 * i);
+        x.x += d.x; x.y += d.y; x.z += d.z; x.w += d.w;
+        if (!rows) st4<float>(hr + 4 * i, x);
+      }
+      v[j] = x;
+      ss += x.x * x.x + x.y * x.y + x.z * x.z + x.w * x.w;
+    }
+  }
+  const float rs = 1.0f / sqrtf(block_sum(ss, red) / (float)H + eps);
+  TO* o = out + (size_t)m * H;
+#pragma unroll
+  for (int j = 0; j < NORM_VEC_MAX; ++j) {
+    const int i = threadIdx.x + 256 * j;
+    if (i < nvec) {
+      const float4 g = ld4<float>(w + 4 * i);
+      st4<TO>(o + 4 * i, float4{(v[j].x * rs) * g.x, (v[j].y * rs) * g.y, (v[j].z * rs) * g.z, (v[j].w * rs) * g.w});
+    }
+  }
+}
+
 extern "C" int qvl_add_rmsnorm(void* h, const void* delta, const void* w, void* out, const void* rows, int M, int H,
                                float eps, int delta_dtype, int out_dtype, hipStream_t stream) {
   if (M <= 0) return QVL_OK;
   if (H <= 0) return QVL_ERR_SHAPE;
   const int threads = H >= 2048 ? 512 : 256;
+  const bool vec = H % 4 == 0 && H <= NORM_VEC_MAX * 4 * 256;
 #define QVL_NORM_CASE(DD, OD, TD, TO)                                                                              \
   if (delta_dtype == DD && out_dtype == OD) {                                                                      \
-    hipLaunchKernelGGL((add_rmsnorm_kernel<TD, TO>), dim3(M), dim3(threads), 0, stream, (float*)h,                 \
-                       (const TD*)delta, (const float*)w, (TO*)out, (const int*)rows, H, eps);                     \
+    if (vec)                                                                                                       \
+      hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TO>), dim3(M), dim3(256), 0, stream, (float*)h,               \
+                         (const TD*)delta, (const float*)w, (TO*)out, (const int*)rows, H, eps);                   \
+    else                                                                                                           \
+      hipLaunchKernelGGL((add_rmsnorm_kernel<TD, TO>), dim3(M), dim3(threads), 0, stream, (float*)h,               \
+                         (const TD*)delta, (const float*)w, (TO*)out, (const int*)rows, H, eps);                   \
     return qvl_launch_status();                                                                                    \
   }
   QVL_NORM_CASE(0, 0, float, float)

@@ -2,6 +2,7 @@
 
 from __future__ import annotations
 
+import os
 from typing import List
 
 from .library import build_library
@@ -25,4 +26,11 @@ LIBRARIES = [
 
 
 def build_everything(force: bool = False, quiet: bool = False) -> List[str]:
-    return [build_library(stem, defines, force=force, quiet=quiet) for stem, defines in LIBRARIES]
+    built = [build_library(stem, defines, force=force, quiet=quiet) for stem, defines in LIBRARIES]
+    # libraries of sources that have changed since are of no use to anyone
+    keep = {os.path.basename(p) for p in built}
+    for directory in {os.path.dirname(p) for p in built}:
+        for name in os.listdir(directory):
+            if name.endswith(".so") and name not in keep:
+                os.remove(os.path.join(directory, name))
+    return built
