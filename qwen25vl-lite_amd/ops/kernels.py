@@ -94,6 +94,8 @@ def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Te
                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``h += delta`` (float32 sum) and return ``rmsnorm(h) * weight`` in ``out_dtype``.
 
+    ``delta`` may be ``[S, N, H]``: partial sums of a product, added in slab order.
+
     With ``rows`` (int32 row indices) only those rows are normalised and ``h`` is not written.
     """
     _dev(h, delta, weight, rows, out)
@@ -101,8 +103,12 @@ def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Te
     n, width = h.shape
     _need(weight.dtype == torch.float32 and weight.shape == (width,) and weight.is_contiguous(),
           "norm weight must be float32 [H]")
+    slabs, slab_stride = 1, 0
     if delta is not None:
-        _need(delta.shape == h.shape and delta.is_contiguous(), "delta must match h's shape")
+        _need(delta.is_contiguous() and tuple(delta.shape[-2:]) == tuple(h.shape) and delta.dim() in (2, 3),
+              "delta must be [N, H] or slabs [S, N, H]")
+        if delta.dim() == 3:
+            slabs, slab_stride = delta.shape[0], delta.stride(0)
     m = n
     if rows is not None:
         _need(rows.dtype == torch.int32 and rows.dim() == 1 and rows.is_contiguous(), "rows must be int32 [M]")
@@ -111,10 +117,11 @@ def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Te
         out = torch.empty((m, width), dtype=out_dtype, device=h.device)
     _need(out.shape == (m, width) and out.dtype == out_dtype and out.is_contiguous(), "out must be [M, H]")
     fn = _fn("elementwise", "qvl_add_rmsnorm",
-             [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr])
+             [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int,
+              ctypes.c_longlong, _c_ptr])
     _check(fn(_ptr(h), _ptr(delta), _ptr(weight), _ptr(out), _ptr(rows), m, width, float(eps),
-              dtype_code(delta.dtype if delta is not None else out_dtype), dtype_code(out_dtype), _stream()),
-           "add_rmsnorm")
+              dtype_code(delta.dtype if delta is not None else out_dtype), dtype_code(out_dtype), slabs, slab_stride,
+              _stream()), "add_rmsnorm")
     return out
 
 

@@ -18,9 +18,11 @@ __all__ = ["linear"]
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
-           out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+           out_dtype: Optional[torch.dtype] = None, allow_slabs: bool = False) -> torch.Tensor:
     """``x [M, K] @ weight[N, K].T (+ bias)``.  ``out_dtype`` float32 is allowed for
-    bfloat16 operands (the products are accumulated in float32 either way)."""
+    bfloat16 operands (the products are accumulated in float32 either way).  With ``allow_slabs``
+    the result may come as partial sums ``[S, M, N]`` whose consumer adds them up (the residual
+    add + norm kernel does); without it the result is always ``[M, N]``."""
     if not x.is_cuda:
         raise kernels.KernelError("linear has no CPU path: its tensors must be on the GPU")
     if x.dtype == torch.float32:
@@ -28,7 +30,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
         raise kernels.KernelError(f"linear: operands {x.dtype}/{weight.dtype} are not built")
     from . import skinny
-    out = skinny.try_linear(x, weight, bias, out_dtype)
+    out = skinny.try_linear(x, weight, bias, out_dtype, allow_slabs)
     if out is not None:
         return out
     if out_dtype == torch.float32:

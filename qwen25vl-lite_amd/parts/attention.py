@@ -101,7 +101,7 @@ class PagedAttention(Mixer):
             group.slot_mapping if write else None, slot.k_cache if write else None, slot.v_cache if write else None,
             self.nq, self.nkv if write else 0, self.hd, group.page_size, out_dtype=self.dtype)
         o = paged_attention(q, slot.k_cache, slot.v_cache, group.block_table, step, self.nq, self.window, self.scale)
-        return linear(o, self.w_out, out_dtype=torch.float32)
+        return linear(o, self.w_out, out_dtype=torch.float32, allow_slabs=True)
 
 
 register_part("mixer", "paged_attention", PagedAttention)

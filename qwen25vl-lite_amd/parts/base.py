@@ -8,7 +8,8 @@ Kinds of parts and what each must provide:
 
 * ``Norm``: ``forward(stream) -> x``.  Folds the stream's pending addend into the float32
   residual and returns the normalised activations in the run dtype.
-* ``Mixer``: ``forward(x, step, slot) -> y`` for ``x`` of ``[N, hidden]``; it may keep keys and
+* ``Mixer``: ``forward(x, step, slot) -> y`` for ``x`` of ``[N, hidden]`` (``y`` may also be
+  partial sums ``[S, N, hidden]``, which the next norm adds up); it may keep keys and
   values in pages (``cache_need()``) and/or a state of fixed size per request
   (``state_need()``), both handed to it through ``slot``.
 * ``FeedForward``: ``forward(x, step) -> y``.
@@ -121,7 +122,7 @@ class ResidualStream:
     norm adds ``pending`` to ``h`` in float32 in the same kernel that normalises."""
 
     h: torch.Tensor                          # float32 [N, hidden]
-    pending: Optional[torch.Tensor] = None   # float32 or run dtype [N, hidden]
+    pending: Optional[torch.Tensor] = None   # [N, hidden], or partial sums [S, N, hidden] added in order
 
 
 class Part:

@@ -46,7 +46,7 @@ class SwiGLU(FeedForward):
 
     def forward(self, x: torch.Tensor, step: StepContext) -> torch.Tensor:
         gate_up = linear(x, self.w_gate_up)
-        return linear(kernels.swiglu(gate_up), self.w_down, out_dtype=torch.float32)
+        return linear(kernels.swiglu(gate_up), self.w_down, out_dtype=torch.float32, allow_slabs=True)
 
 
 register_part("ffn", "swiglu", SwiGLU)

@@ -43,6 +43,12 @@ def test_add_rmsnorm(width, delta_dtype, out_dtype):
     assert out.dtype == out_dtype
     assert torch.allclose(out.float().cpu(), want, **_tol(out_dtype))
     assert torch.allclose(hd.cpu(), total, atol=1e-6), "the sum is written back in float32"
+    if delta is not None and delta_dtype == torch.float32:
+        # partial sums in slabs are added in order
+        parts = torch.stack([delta * 0.25, delta * 0.5, delta * 0.25])
+        hd = h.cuda()
+        out = kernels.add_rmsnorm(hd, parts.cuda(), w.cuda(), eps, out_dtype)
+        assert torch.allclose(out.float().cpu(), want, **_tol(out_dtype)) and torch.allclose(hd.cpu(), total, atol=1e-5)
     # selected rows: h stays as it was
     hd = h.cuda()
     rows = torch.tensor([4, 0, 4], dtype=torch.int32).cuda()
@@ -214,7 +220,7 @@ def test_gemm_f32_is_exact_and_row_independent(m, n, k):
     assert torch.equal(alone[0], out[m // 2])
 
 
-@pytest.mark.parametrize("m, n, k", [(1, 509, 144), (8, 300, 200), (16, 17, 8), (17, 1000, 4104), (31, 130, 352),
+@pytest.mark.parametrize("m, n, k", [(1, 509, 144), (8, 300, 200), (16, 17, 8), (9, 100, 8200), (17, 1000, 4104), (31, 130, 352),
                                      (64, 509, 3584), (5, 40, 100), (300, 64, 1000)])
 def test_linear_bfloat16(m, n, k):
     """Few rows go through the skinny matrix-core kernel (inner sizes in steps of 8), the rest
@@ -227,6 +233,12 @@ def test_linear_bfloat16(m, n, k):
     want = x.float() @ w.float().T
     took = skinny.try_linear(x.cuda(), w.cuda(), None, torch.float32)
     assert (took is not None) == (m <= 32 and k % 8 == 0)
+    if m <= 16 and k % 8 == 0:
+        # an inner size above 4096 comes as partial sums in slabs, if the caller takes them
+        slabs = skinny.try_linear(x.cuda(), w.cuda(), None, torch.float32, allow_slabs=True)
+        assert slabs.dim() == (3 if k > 4096 else 2)
+        total = slabs.sum(0) if slabs.dim() == 3 else slabs
+        assert torch.allclose(total.cpu(), want, atol=2e-3, rtol=2e-3)
     out32 = linear(x.cuda(), w.cuda(), out_dtype=torch.float32)
     assert out32.dtype == torch.float32 and torch.allclose(out32.cpu(), want, atol=2e-3, rtol=2e-3)
     out16 = linear(x.cuda(), w.cuda())
