@@ -63,12 +63,15 @@ struct BlockRegs {
   bf16x8_t v[NT];
 };
 
+// CT: column tiles (of 16 columns) a wave carries through the walk; every key block it loads is
+// used for all of them.
+template <int CT>
 struct Walk {
   const bf16_t* kc;
   const bf16_t* vc;
   const int* bt;  // this request's row of the block table
   int max_key, nkv, kvh, ps;
-  int my_lo, my_p, key_begin, key_end;
+  int my_lo[CT], my_p[CT], key_begin, key_end;
   float scale_log2;
   int lg, r;
 
@@ -101,54 +104,58 @@ struct Walk {
     for (int dt = 0; dt < NT; ++dt) rg.v[dt] = load8(vbase + (size_t)(dt * 16 + r) * ps);
   }
 
-  __device__ __forceinline__ void compute(int kb, const bf16x8_t* qb, const BlockRegs& rg, TileState& st) const {
+  __device__ __forceinline__ void compute(int kb, const bf16x8_t (*qb)[KS], const BlockRegs& rg, TileState* sts) const {
     const int key0 = kb << 5;
-    f32x4_t s[2];
 #pragma unroll
-    for (int b = 0; b < 2; ++b) {
-      f32x4_t a = {0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < CT; ++t) {
+      TileState& st = sts[t];
+      f32x4_t s[2];
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(rg.k[b][ks], qb[ks], a, 0, 0, 0);
-      s[b] = a;
-    }
-    // mask and online softmax; this lane holds keys key0 + 8*lg + j of column r
-    float sv[8];
-    float mloc = -INFINITY;
+      for (int b = 0; b < 2; ++b) {
+        f32x4_t a = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int key = key0 + 8 * lg + j;
-      const float raw = (j < 4) ? s[0][j] : s[1][j - 4];
-      const bool ok = key >= my_lo && key <= my_p && key >= key_begin && key <= key_end;
-      sv[j] = ok ? raw * scale_log2 : -INFINITY;
-      mloc = fmaxf(mloc, sv[j]);
-    }
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 16, QVL_WAVE));
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, QVL_WAVE));
-    const float m_new = fmaxf(st.m, mloc);
-    float alpha = 1.f, psum = 0.f;
-    float pv[8];
-    if (m_new == -INFINITY) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) pv[j] = 0.f;
-    } else {
-      alpha = exp2f(st.m - m_new);
+        for (int ks = 0; ks < KS; ++ks) a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(rg.k[b][ks], qb[t][ks], a, 0, 0, 0);
+        s[b] = a;
+      }
+      // mask and online softmax; this lane holds keys key0 + 8*lg + j of column r
+      float sv[8];
+      float mloc = -INFINITY;
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        pv[j] = exp2f(sv[j] - m_new);
-        psum += pv[j];
+        const int key = key0 + 8 * lg + j;
+        const float raw = (j < 4) ? s[0][j] : s[1][j - 4];
+        const bool ok = key >= my_lo[t] && key <= my_p[t] && key >= key_begin && key <= key_end;
+        sv[j] = ok ? raw * scale_log2 : -INFINITY;
+        mloc = fmaxf(mloc, sv[j]);
       }
-    }
-    psum += __shfl_xor(psum, 16, QVL_WAVE);
-    psum += __shfl_xor(psum, 32, QVL_WAVE);
-    st.l = st.l * alpha + psum;
-    st.m = m_new;
-    u32x4_t packed = {pack2(pv[0], pv[1]), pack2(pv[2], pv[3]), pack2(pv[4], pv[5]), pack2(pv[6], pv[7])};
-    const bf16x8_t pb = __builtin_bit_cast(bf16x8_t, packed);
+      mloc = fmaxf(mloc, __shfl_xor(mloc, 16, QVL_WAVE));
+      mloc = fmaxf(mloc, __shfl_xor(mloc, 32, QVL_WAVE));
+      const float m_new = fmaxf(st.m, mloc);
+      float alpha = 1.f, psum = 0.f;
+      float pv[8];
+      if (m_new == -INFINITY) {
 #pragma unroll
-    for (int dt = 0; dt < NT; ++dt) {
-      f32x4_t o = st.acc[dt];
-      o[0] *= alpha; o[1] *= alpha; o[2] *= alpha; o[3] *= alpha;
-      st.acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(rg.v[dt], pb, o, 0, 0, 0);
+        for (int j = 0; j < 8; ++j) pv[j] = 0.f;
+      } else {
+        alpha = exp2f(st.m - m_new);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          pv[j] = exp2f(sv[j] - m_new);
+          psum += pv[j];
+        }
+      }
+      psum += __shfl_xor(psum, 16, QVL_WAVE);
+      psum += __shfl_xor(psum, 32, QVL_WAVE);
+      st.l = st.l * alpha + psum;
+      st.m = m_new;
+      u32x4_t packed = {pack2(pv[0], pv[1]), pack2(pv[2], pv[3]), pack2(pv[4], pv[5]), pack2(pv[6], pv[7])};
+      const bf16x8_t pb = __builtin_bit_cast(bf16x8_t, packed);
+#pragma unroll
+      for (int dt = 0; dt < NT; ++dt) {
+        f32x4_t o = st.acc[dt];
+        o[0] *= alpha; o[1] *= alpha; o[2] *= alpha; o[3] *= alpha;
+        st.acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(rg.v[dt], pb, o, 0, 0, 0);
+      }
     }
   }
 };
@@ -156,15 +163,18 @@ struct Walk {
 // Walk the 32-key blocks first, first + stride, ... that overlap keys [key_begin, key_end]
 // (inclusive, absolute) of one tile.  The loads of the next block and the page lookups of the one
 // after are issued before the current block is computed, so a wave always has a block in flight.
+template <int CT>
 __device__ __forceinline__ void attend(const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
                                        const int* __restrict__ bt, int table_width, int nkv, int kvh, int ps,
-                                       const bf16x8_t* qb, int my_lo, int my_p, float scale_log2, int key_begin,
-                                       int key_end, int kb_offset, int kb_stride, TileState& st) {
+                                       const bf16x8_t (*qb)[KS], const int* my_lo, const int* my_p, float scale_log2,
+                                       int key_begin, int key_end, int kb_offset, int kb_stride, TileState* st) {
   const int lane = threadIdx.x & 63;
-  Walk w;
+  Walk<CT> w;
   w.kc = kc; w.vc = vc; w.bt = bt;
   w.max_key = table_width * ps - 1; w.nkv = nkv; w.kvh = kvh; w.ps = ps;
-  w.my_lo = my_lo; w.my_p = my_p; w.key_begin = key_begin; w.key_end = key_end;
+#pragma unroll
+  for (int t = 0; t < CT; ++t) { w.my_lo[t] = my_lo[t]; w.my_p[t] = my_p[t]; }
+  w.key_begin = key_begin; w.key_end = key_end;
   w.scale_log2 = scale_log2; w.lg = lane >> 4; w.r = lane & 15;
   const int s = kb_stride;
   int kb = (key_begin >> 5) + kb_offset;
@@ -229,6 +239,17 @@ __device__ __forceinline__ void load_q(const bf16_t* __restrict__ q, int nq, con
   }
 }
 
+// Column tiles per wave in the kernel for many tiles: every key block a wave loads serves two tiles.
+#define TILE_CT 2
+
+__device__ __forceinline__ void init_state(TileState& st) {
+  st.m = -INFINITY;
+  st.l = 0.f;
+#pragma unroll
+  for (int dt = 0; dt < NT; ++dt) st.acc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+}
+
+// tile_ct counts in units of TILE_CT column tiles here.
 __global__ __launch_bounds__(256) void attn_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc,
                                                         const bf16_t* __restrict__ vc, const int* __restrict__ bt,
                                                         int table_width, const int* __restrict__ cu_q,
@@ -240,28 +261,43 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const bf16_t* __restrict
   const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (item >= num_tiles) return;
   const int kvh = blockIdx.y, g = nq / nkv;
-  const int r = tile_req[item], ct = tile_ct[item];
-  const TileInfo t = tile_info(cu_q, ctx_len, r, ct, g, kvh, window);
-  bf16x8_t qb[KS];
-  load_q(q, nq, t, qb);
-  TileState st;
-  st.m = -INFINITY;
-  st.l = 0.f;
+  const int r = tile_req[item], ct0 = tile_ct[item] * TILE_CT;
+  const int ncols = (cu_q[r + 1] - cu_q[r]) * g;
+  TileInfo t[TILE_CT];
+  bf16x8_t qb[TILE_CT][KS];
+  TileState st[TILE_CT];
+  int my_lo[TILE_CT], my_p[TILE_CT];
+  int lo = 0x7fffffff, hi = -1;
 #pragma unroll
-  for (int dt = 0; dt < NT; ++dt) st.acc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  attend(kc, vc, bt + (size_t)r * table_width, table_width, nkv, kvh, ps, qb, t.my_lo, t.my_p, scale * LOG2E,
-         t.lo_tile, t.hi_tile, 0, 1, st);
-  if (!t.valid) return;
+  for (int i = 0; i < TILE_CT; ++i) {
+    const bool exists = (ct0 + i) * 16 < ncols;   // the last pair of a request may have one tile only
+    t[i] = tile_info(cu_q, ctx_len, r, exists ? ct0 + i : ct0, g, kvh, window);
+    if (!exists) { t[i].valid = false; t[i].my_p = -1; }
+    load_q(q, nq, t[i], qb[i]);
+    init_state(st[i]);
+    my_lo[i] = t[i].my_lo;
+    my_p[i] = t[i].my_p;
+    if (exists) {
+      lo = t[i].lo_tile < lo ? t[i].lo_tile : lo;
+      hi = t[i].hi_tile > hi ? t[i].hi_tile : hi;
+    }
+  }
+  attend<TILE_CT>(kc, vc, bt + (size_t)r * table_width, table_width, nkv, kvh, ps, qb, my_lo, my_p, scale * LOG2E, lo,
+                  hi, 0, 1, st);
   const int lg = (threadIdx.x & 63) >> 4;
-  const float inv = 1.0f / st.l;
-  bf16_t* orow = out + ((size_t)t.token * nq + t.head) * HD;
 #pragma unroll
-  for (int dt = 0; dt < NT; ++dt) {
-    const int d = dt * 16 + 4 * lg;
-    uint2 w;
-    w.x = pack2(st.acc[dt][0] * inv, st.acc[dt][1] * inv);
-    w.y = pack2(st.acc[dt][2] * inv, st.acc[dt][3] * inv);
-    *reinterpret_cast<uint2*>(orow + d) = w;
+  for (int i = 0; i < TILE_CT; ++i) {
+    if (!t[i].valid) continue;
+    const float inv = 1.0f / st[i].l;
+    bf16_t* orow = out + ((size_t)t[i].token * nq + t[i].head) * HD;
+#pragma unroll
+    for (int dt = 0; dt < NT; ++dt) {
+      const int d = dt * 16 + 4 * lg;
+      uint2 w;
+      w.x = pack2(st[i].acc[dt][0] * inv, st[i].acc[dt][1] * inv);
+      w.y = pack2(st[i].acc[dt][2] * inv, st[i].acc[dt][3] * inv);
+      *reinterpret_cast<uint2*>(orow + d) = w;
+    }
   }
 }
 
@@ -299,15 +335,12 @@ __global__ __launch_bounds__(64 * COOP_WAVES) void attn_mfma_coop_kernel(
     first = first > t.lo_tile ? first : t.lo_tile;
   }
   TileState st;
-  st.m = -INFINITY;
-  st.l = 0.f;
-#pragma unroll
-  for (int dt = 0; dt < NT; ++dt) st.acc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  init_state(st);
   if (first <= last) {
-    bf16x8_t qb[KS];
-    load_q(q, nq, t, qb);
-    attend(kc, vc, bt + (size_t)r * table_width, table_width, nkv, kvh, ps, qb, t.my_lo, t.my_p, scale * LOG2E,
-           first, last, wave, COOP_WAVES, st);
+    bf16x8_t qb[1][KS];
+    load_q(q, nq, t, qb[0]);
+    attend<1>(kc, vc, bt + (size_t)r * table_width, table_width, nkv, kvh, ps, qb, &t.my_lo, &t.my_p, scale * LOG2E,
+              first, last, wave, COOP_WAVES, &st);
   }
   // every wave leaves its column sums in LDS: column c, channels dt*16 + 4*lg .. +3, then m and l
   float* mine = &sm[wave][c * PART_COLS];
@@ -396,6 +429,8 @@ static int check_common(int num_tiles, int nq, int nkv, int ps, int table_width)
 }
 
 extern "C" int qvl_attn_mfma_head_dim() { return HD; }
+// Column tiles per entry of the tile list that qvl_attn_mfma expects (qvl_attn_mfma_coop: 1).
+extern "C" int qvl_attn_mfma_tile_ct() { return TILE_CT; }
 
 extern "C" int qvl_attn_mfma(const void* q, const void* kc, const void* vc, const void* bt, int table_width,
                              const void* cu_q, const void* ctx_len, const void* tile_req, const void* tile_ct,

@@ -252,6 +252,30 @@ __global__ void swiglu_kernel(const T* __restrict__ x, T* __restrict__ out, int 
   stf<T>(out + (size_t)n * I + i, (g / (1.0f + expf(-g))) * u);
 }
 
+// bfloat16 rows whose width is a multiple of 8: eight values per thread, 16-byte loads and stores.
+__global__ __launch_bounds__(256) void swiglu_bf16x8_kernel(const bf16_t* __restrict__ x, bf16_t* __restrict__ out,
+                                                            int I, long long total8) {
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  const int per_row = I >> 3;
+  for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total8;
+       idx += (long long)gridDim.x * blockDim.x) {
+    const long long n = idx / per_row;
+    const int c = (int)(idx - n * per_row) << 3;
+    const bf16_t* row = x + (size_t)n * 2 * I;
+    const u32x4 gv = *reinterpret_cast<const u32x4*>(row + c);
+    const u32x4 uv = *reinterpret_cast<const u32x4*>(row + I + c);
+    u32x4 o;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float g0 = __uint_as_float(gv[k] << 16), g1 = __uint_as_float(gv[k] & 0xffff0000u);
+      const float u0 = __uint_as_float(uv[k] << 16), u1 = __uint_as_float(uv[k] & 0xffff0000u);
+      const float a0 = (g0 / (1.0f + expf(-g0))) * u0, a1 = (g1 / (1.0f + expf(-g1))) * u1;
+      o[k] = (uint32_t)f32_to_bf16(a0) | ((uint32_t)f32_to_bf16(a1) << 16);
+    }
+    *reinterpret_cast<u32x4*>(out + (size_t)n * I + c) = o;
+  }
+}
+
 extern "C" int qvl_swiglu(const void* x, void* out, int N, int I, int dtype, hipStream_t stream) {
   if (N <= 0) return QVL_OK;
   if (I <= 0) return QVL_ERR_SHAPE;
@@ -259,7 +283,13 @@ extern "C" int qvl_swiglu(const void* x, void* out, int N, int I, int dtype, hip
   const dim3 grid((I + 255) / 256, N);
   if (dtype == 0)
     hipLaunchKernelGGL(swiglu_kernel<float>, grid, dim3(256), 0, stream, (const float*)x, (float*)out, I);
-  else if (dtype == 1)
+  else if (dtype == 1 && I % 8 == 0 && (((uintptr_t)x | (uintptr_t)out) & 15) == 0) {
+    const long long total8 = (long long)N * (I >> 3);
+    long long blocks = (total8 + 255) / 256;
+    blocks = blocks > 8192 ? 8192 : blocks;
+    hipLaunchKernelGGL(swiglu_bf16x8_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (const bf16_t*)x,
+                       (bf16_t*)out, I, total8);
+  } else if (dtype == 1)
     hipLaunchKernelGGL(swiglu_kernel<bf16_t>, grid, dim3(256), 0, stream, (const bf16_t*)x, (bf16_t*)out, I);
   else
     return QVL_ERR_DTYPE;

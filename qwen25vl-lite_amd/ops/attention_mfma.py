@@ -28,10 +28,13 @@ def supports(head_dim: int, dtype: torch.dtype) -> bool:
     return dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= _MAX_HD
 
 
-def tiles_for(cu_q, group: int) -> Tuple[np.ndarray, np.ndarray]:
-    """``(tile_req, tile_ct)``: for request r with q tokens, ceil(q * group / 16) tiles."""
+TILE_CT = 2   # column tiles a wave carries in the kernel for many tiles (TILE_CT in the source)
+
+
+def tiles_for(cu_q, group: int, tile_ct: int = 1) -> Tuple[np.ndarray, np.ndarray]:
+    """``(tile_req, tile_ct)``: for request r with q tokens, ceil(q * group / (16 * tile_ct)) entries."""
     q = np.diff(np.asarray(cu_q, dtype=np.int64))
-    counts = (q * group + 15) // 16
+    counts = (q * group + 16 * tile_ct - 1) // (16 * tile_ct)
     req = np.repeat(np.arange(len(q), dtype=np.int32), counts)
     starts = np.cumsum(counts) - counts
     ct = (np.arange(int(counts.sum()), dtype=np.int64) - np.repeat(starts, counts)).astype(np.int32)
@@ -53,11 +56,11 @@ def plan_splits(num_tiles: int, nkv: int, max_ctx: int) -> Tuple[str, int, int]:
     return "coop", (max_ctx + 31 + per - 1) // per, per
 
 
-def _step_tiles(step, group: int, device):
+def _step_tiles(step, group: int, tile_ct: int, device):
     cache = step.derived
-    key = ("tiles", group)
+    key = ("tiles", group, tile_ct)
     if key not in cache:
-        req, ct = tiles_for(step.cu_q_host, group)
+        req, ct = tiles_for(step.cu_q_host, group, tile_ct)
         both = torch.from_numpy(np.concatenate([req, ct])).to(device, non_blocking=True)
         cache[key] = (both[:len(req)], both[len(req):], len(req))
     return cache[key]
@@ -76,10 +79,12 @@ def try_attention(q, k_cache, v_cache, block_table, step, num_q_heads: int, wind
     _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous()
           and block_table.shape[0] == step.num_reqs, "block_table must be int32 [R, width]")
     _need(nq % nkv == 0, "query heads must be a multiple of key/value heads")
-    tile_req, tile_ct, num_tiles = _step_tiles(step, nq // nkv, q.device)
+    tile_req, tile_ct, num_tiles = _step_tiles(step, nq // nkv, 1, q.device)
     out = torch.empty_like(q)
     defines = {"HD": hd}
     kind, nsplit, per = plan_splits(num_tiles, nkv, step.max_ctx_len)
+    if kind == "tile":
+        tile_req, tile_ct, num_tiles = _step_tiles(step, nq // nkv, TILE_CT, q.device)
     common = [_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(step.cu_q),
               _ptr(step.ctx_len), _ptr(tile_req), _ptr(tile_ct), num_tiles, _ptr(out)]
     if kind == "tile":

@@ -194,11 +194,12 @@ def test_paged_attention_matrix_cores(nq, nkv, hd, window, split, monkeypatch):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_swiglu(dtype):
+@pytest.mark.parametrize("rows, inter", [(7, 353), (5, 352), (70, 18944)])
+def test_swiglu(dtype, rows, inter):
     from qwen25vl_lite_amd.ops import kernels
     torch.manual_seed(3)
-    x = (torch.randn(7, 2 * 353) * 3).to(dtype)
-    want = torch.nn.functional.silu(x[:, :353].float()) * x[:, 353:].float()
+    x = (torch.randn(rows, 2 * inter) * 3).to(dtype)
+    want = torch.nn.functional.silu(x[:, :inter].float()) * x[:, inter:].float()
     out = kernels.swiglu(x.cuda())
     assert torch.allclose(out.float().cpu(), want, **_tol(dtype))
 
