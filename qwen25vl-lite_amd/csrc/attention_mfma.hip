@@ -44,8 +44,12 @@ __device__ __forceinline__ bf16x8_t zero8() {
   u32x4_t z = {0u, 0u, 0u, 0u};
   return __builtin_bit_cast(bf16x8_t, z);
 }
+// Two floats to two bfloat16 (round to nearest even) in one word; the compiler uses the packed
+// hardware conversion of gfx950.
 __device__ __forceinline__ uint32_t pack2(float a, float b) {
-  return (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  bf16x2_t v = {(__bf16)a, (__bf16)b};
+  return __builtin_bit_cast(uint32_t, v);
 }
 
 struct TileState {
@@ -72,6 +76,7 @@ struct Walk {
   const int* bt;  // this request's row of the block table
   int max_key, nkv, kvh, ps;
   int my_lo[CT], my_p[CT], key_begin, key_end;
+  int all_lo, all_hi;  // keys all_lo .. all_hi are seen by every column of the wave
   float scale_log2;
   int lg, r;
 
@@ -106,6 +111,7 @@ struct Walk {
 
   __device__ __forceinline__ void compute(int kb, const bf16x8_t (*qb)[KS], const BlockRegs& rg, TileState* sts) const {
     const int key0 = kb << 5;
+    const bool interior = key0 >= all_lo && key0 + 31 <= all_hi;
 #pragma unroll
     for (int t = 0; t < CT; ++t) {
       TileState& st = sts[t];
@@ -117,16 +123,25 @@ struct Walk {
         for (int ks = 0; ks < KS; ++ks) a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(rg.k[b][ks], qb[t][ks], a, 0, 0, 0);
         s[b] = a;
       }
-      // mask and online softmax; this lane holds keys key0 + 8*lg + j of column r
+      // mask and online softmax; this lane holds keys key0 + 8*lg + j of column r.  A block that
+      // lies wholly inside what every column of the wave sees needs no mask.
       float sv[8];
       float mloc = -INFINITY;
+      if (interior) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int key = key0 + 8 * lg + j;
-        const float raw = (j < 4) ? s[0][j] : s[1][j - 4];
-        const bool ok = key >= my_lo[t] && key <= my_p[t] && key >= key_begin && key <= key_end;
-        sv[j] = ok ? raw * scale_log2 : -INFINITY;
-        mloc = fmaxf(mloc, sv[j]);
+        for (int j = 0; j < 8; ++j) {
+          sv[j] = ((j < 4) ? s[0][j] : s[1][j - 4]) * scale_log2;
+          mloc = fmaxf(mloc, sv[j]);
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int key = key0 + 8 * lg + j;
+          const float raw = (j < 4) ? s[0][j] : s[1][j - 4];
+          const bool ok = key >= my_lo[t] && key <= my_p[t] && key >= key_begin && key <= key_end;
+          sv[j] = ok ? raw * scale_log2 : -INFINITY;
+          mloc = fmaxf(mloc, sv[j]);
+        }
       }
       mloc = fmaxf(mloc, __shfl_xor(mloc, 16, QVL_WAVE));
       mloc = fmaxf(mloc, __shfl_xor(mloc, 32, QVL_WAVE));
@@ -137,10 +152,10 @@ struct Walk {
 #pragma unroll
         for (int j = 0; j < 8; ++j) pv[j] = 0.f;
       } else {
-        alpha = exp2f(st.m - m_new);
+        alpha = __builtin_amdgcn_exp2f(st.m - m_new);
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          pv[j] = exp2f(sv[j] - m_new);
+          pv[j] = __builtin_amdgcn_exp2f(sv[j] - m_new);
           psum += pv[j];
         }
       }
@@ -148,14 +163,22 @@ struct Walk {
       psum += __shfl_xor(psum, 32, QVL_WAVE);
       st.l = st.l * alpha + psum;
       st.m = m_new;
+      // the running maximum rarely moves after the first blocks: skip the rescaling when no
+      // column of the wave needs it
+      const bool rescale = __any(alpha != 1.f);
       u32x4_t packed = {pack2(pv[0], pv[1]), pack2(pv[2], pv[3]), pack2(pv[4], pv[5]), pack2(pv[6], pv[7])};
       const bf16x8_t pb = __builtin_bit_cast(bf16x8_t, packed);
+      if (rescale) {
 #pragma unroll
-      for (int dt = 0; dt < NT; ++dt) {
-        f32x4_t o = st.acc[dt];
-        o[0] *= alpha; o[1] *= alpha; o[2] *= alpha; o[3] *= alpha;
-        st.acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(rg.v[dt], pb, o, 0, 0, 0);
+        for (int dt = 0; dt < NT; ++dt) {
+          f32x4_t o = st.acc[dt];
+          o[0] *= alpha; o[1] *= alpha; o[2] *= alpha; o[3] *= alpha;
+          st.acc[dt] = o;
+        }
       }
+#pragma unroll
+      for (int dt = 0; dt < NT; ++dt)
+        st.acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(rg.v[dt], pb, st.acc[dt], 0, 0, 0);
     }
   }
 };
@@ -176,6 +199,23 @@ __device__ __forceinline__ void attend(const bf16_t* __restrict__ kc, const bf16
   for (int t = 0; t < CT; ++t) { w.my_lo[t] = my_lo[t]; w.my_p[t] = my_p[t]; }
   w.key_begin = key_begin; w.key_end = key_end;
   w.scale_log2 = scale_log2; w.lg = lane >> 4; w.r = lane & 15;
+  {  // the range every column sees: largest first key and smallest last key over all lanes and tiles
+    int lo = key_begin, hi = key_end;
+#pragma unroll
+    for (int t = 0; t < CT; ++t) {
+      if (my_p[t] >= 0) {  // a lane without a column computes on zeros and stores nothing
+        lo = max(lo, my_lo[t]);
+        hi = min(hi, my_p[t]);
+      }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      lo = max(lo, __shfl_xor(lo, o, QVL_WAVE));
+      hi = min(hi, __shfl_xor(hi, o, QVL_WAVE));
+    }
+    w.all_lo = lo;
+    w.all_hi = hi;
+  }
   const int s = kb_stride;
   int kb = (key_begin >> 5) + kb_offset;
 #define LIVE(x) (((x) << 5) <= key_end)
