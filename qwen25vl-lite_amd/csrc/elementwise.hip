@@ -34,8 +34,7 @@ extern "C" int qvl_embed_gather(const void* ids, const void* table, void* out, i
 
 // ---------------------------------------------------------------------------------------
 // Residual add + RMSNorm  (reference layers.py:27-31, text.py:196-205)
-//   v = h[row] + delta[row]            (delta optional; the sum is float32; delta may come as several
-//                                       slabs [slab][row], partial sums of a product, added in slab order)
+//   v = h[row] + delta[row]            (delta optional; the sum is float32)
 //   h[row] = v                         (unless `rows` selects rows: then h is left alone)
 //   out[m] = v * (1/sqrt(mean(v^2) + eps)) * w
 // One block per row; the reduction order depends on H only, so a row's result does not
@@ -43,8 +42,7 @@ extern "C" int qvl_embed_gather(const void* ids, const void* table, void* out, i
 // ---------------------------------------------------------------------------------------
 template <typename TD, typename TO>
 __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__ delta, const float* __restrict__ w,
-                                   TO* __restrict__ out, const int* __restrict__ rows, int H, float eps, int slabs,
-                                   size_t slab_stride) {
+                                   TO* __restrict__ out, const int* __restrict__ rows, int H, float eps) {
   __shared__ float red[17];
   const int m = blockIdx.x;
   const int row = rows ? rows[m] : m;
@@ -53,8 +51,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__
   float ss = 0.f;
   for (int i = threadIdx.x; i < H; i += blockDim.x) {
     float v = hr[i];
-    if (dr)
-      for (int sl = 0; sl < slabs; ++sl) v += ldf<TD>(dr + sl * slab_stride + i);
+    if (dr) v += ldf<TD>(dr + i);
     ss += v * v;
     if (dr && !rows) hr[i] = v;
   }
@@ -63,8 +60,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__
   TO* o = out + (size_t)m * H;
   for (int i = threadIdx.x; i < H; i += blockDim.x) {
     float v = hr[i];
-    if (dr && rows)
-      for (int sl = 0; sl < slabs; ++sl) v += ldf<TD>(dr + sl * slab_stride + i);
+    if (dr && rows) v += ldf<TD>(dr + i);
     stf<TO>(o + i, (v * rs) * w[i]);
   }
 }
@@ -92,8 +88,7 @@ template <> __device__ __forceinline__ void st4<bf16_t>(bf16_t* p, float4 v) {
 template <typename TD, typename TO>
 __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict__ h, const TD* __restrict__ delta,
                                                               const float* __restrict__ w, TO* __restrict__ out,
-                                                              const int* __restrict__ rows, int H, float eps,
-                                                              int slabs, size_t slab_stride) {
+                                                              const int* __restrict__ rows, int H, float eps) {
   __shared__ float red[17];
   const int m = blockIdx.x;
   const int row = rows ? rows[m] : m;
@@ -108,10 +103,8 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
     if (i < nvec) {
       float4 x = ld4<float>(hr + 4 * i);
       if (dr) {
-        for (int sl = 0; sl < slabs; ++sl) {
-          const float4 d = ld4<TD>(dr + sl * slab_stride + 4 * i);
-          x.x += d.x; x.y += d.y; x.z += d.z; x.w += d.w;
-        }
+        const float4 d = ld4<TD>(dr + 4 * i);
+        x.x += d.x; x.y += d.y; x.z += d.z; x.w += d.w;
         if (!rows) st4<float>(hr + 4 * i, x);
       }
       v[j] = x;
@@ -131,22 +124,19 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
 }
 
 extern "C" int qvl_add_rmsnorm(void* h, const void* delta, const void* w, void* out, const void* rows, int M, int H,
-                               float eps, int delta_dtype, int out_dtype, int slabs, long long slab_stride,
-                               hipStream_t stream) {
+                               float eps, int delta_dtype, int out_dtype, hipStream_t stream) {
   if (M <= 0) return QVL_OK;
-  if (H <= 0 || slabs < 1 || (slabs > 1 && slab_stride <= 0)) return QVL_ERR_SHAPE;
+  if (H <= 0) return QVL_ERR_SHAPE;
   const int threads = H >= 2048 ? 512 : 256;
   const bool vec = H % 4 == 0 && H <= NORM_VEC_MAX * 4 * 256;
 #define QVL_NORM_CASE(DD, OD, TD, TO)                                                                              \
   if (delta_dtype == DD && out_dtype == OD) {                                                                      \
     if (vec)                                                                                                       \
       hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TO>), dim3(M), dim3(256), 0, stream, (float*)h,               \
-                         (const TD*)delta, (const float*)w, (TO*)out, (const int*)rows, H, eps, slabs,             \
-                         (size_t)slab_stride);                                                                     \
+                         (const TD*)delta, (const float*)w, (TO*)out, (const int*)rows, H, eps);                   \
     else                                                                                                           \
       hipLaunchKernelGGL((add_rmsnorm_kernel<TD, TO>), dim3(M), dim3(threads), 0, stream, (float*)h,               \
-                         (const TD*)delta, (const float*)w, (TO*)out, (const int*)rows, H, eps, slabs,             \
-                         (size_t)slab_stride);                                                                     \
+                         (const TD*)delta, (const float*)w, (TO*)out, (const int*)rows, H, eps);                   \
     return qvl_launch_status();                                                                                    \
   }
   QVL_NORM_CASE(0, 0, float, float)
@@ -239,22 +229,26 @@ extern "C" int qvl_rope_kv_write(const void* x, int x_stride, const void* bias, 
 }
 
 // ---------------------------------------------------------------------------------------
-// SwiGLU: out[n, i] = silu(x[n, i]) * x[n, I + i],  silu(z) = z / (1 + exp(-z))
-// (reference text.py:66)
+// SwiGLU: out[n, i] = silu(gate[n, i]) * up[n, i],  silu(z) = z / (1 + exp(-z))  (reference text.py:66)
+// x[n] holds gate and up: plain, gate in columns 0..I-1 and up in I..2I-1; grouped, alternating
+// groups of 8 gate columns and 8 up columns (feature i: gate at 16 (i/8) + i%8, up 8 further),
+// the layout that lets the product before it apply the activation to a 16-row tile by itself.
 // ---------------------------------------------------------------------------------------
 template <typename T>
-__global__ void swiglu_kernel(const T* __restrict__ x, T* __restrict__ out, int I) {
+__global__ void swiglu_kernel(const T* __restrict__ x, T* __restrict__ out, int I, int grouped) {
   const int n = blockIdx.y;
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= I) return;
   const T* row = x + (size_t)n * 2 * I;
-  const float g = ldf<T>(row + i), u = ldf<T>(row + I + i);
+  const int gc = grouped ? 16 * (i >> 3) + (i & 7) : i;
+  const int uc = grouped ? gc + 8 : I + i;
+  const float g = ldf<T>(row + gc), u = ldf<T>(row + uc);
   stf<T>(out + (size_t)n * I + i, (g / (1.0f + expf(-g))) * u);
 }
 
 // bfloat16 rows whose width is a multiple of 8: eight values per thread, 16-byte loads and stores.
 __global__ __launch_bounds__(256) void swiglu_bf16x8_kernel(const bf16_t* __restrict__ x, bf16_t* __restrict__ out,
-                                                            int I, long long total8) {
+                                                            int I, long long total8, int grouped) {
   typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
   const int per_row = I >> 3;
   for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total8;
@@ -262,8 +256,8 @@ __global__ __launch_bounds__(256) void swiglu_bf16x8_kernel(const bf16_t* __rest
     const long long n = idx / per_row;
     const int c = (int)(idx - n * per_row) << 3;
     const bf16_t* row = x + (size_t)n * 2 * I;
-    const u32x4 gv = *reinterpret_cast<const u32x4*>(row + c);
-    const u32x4 uv = *reinterpret_cast<const u32x4*>(row + I + c);
+    const u32x4 gv = *reinterpret_cast<const u32x4*>(row + (grouped ? 2 * c : c));
+    const u32x4 uv = *reinterpret_cast<const u32x4*>(row + (grouped ? 2 * c + 8 : I + c));
     u32x4 o;
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
@@ -276,21 +270,22 @@ __global__ __launch_bounds__(256) void swiglu_bf16x8_kernel(const bf16_t* __rest
   }
 }
 
-extern "C" int qvl_swiglu(const void* x, void* out, int N, int I, int dtype, hipStream_t stream) {
+extern "C" int qvl_swiglu(const void* x, void* out, int N, int I, int dtype, int grouped, hipStream_t stream) {
   if (N <= 0) return QVL_OK;
-  if (I <= 0) return QVL_ERR_SHAPE;
+  if (I <= 0 || (grouped && I % 8)) return QVL_ERR_SHAPE;
   if (N > 65535) return QVL_ERR_LIMIT;
   const dim3 grid((I + 255) / 256, N);
   if (dtype == 0)
-    hipLaunchKernelGGL(swiglu_kernel<float>, grid, dim3(256), 0, stream, (const float*)x, (float*)out, I);
+    hipLaunchKernelGGL(swiglu_kernel<float>, grid, dim3(256), 0, stream, (const float*)x, (float*)out, I, grouped);
   else if (dtype == 1 && I % 8 == 0 && (((uintptr_t)x | (uintptr_t)out) & 15) == 0) {
     const long long total8 = (long long)N * (I >> 3);
     long long blocks = (total8 + 255) / 256;
     blocks = blocks > 8192 ? 8192 : blocks;
     hipLaunchKernelGGL(swiglu_bf16x8_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (const bf16_t*)x,
-                       (bf16_t*)out, I, total8);
+                       (bf16_t*)out, I, total8, grouped);
   } else if (dtype == 1)
-    hipLaunchKernelGGL(swiglu_kernel<bf16_t>, grid, dim3(256), 0, stream, (const bf16_t*)x, (bf16_t*)out, I);
+    hipLaunchKernelGGL(swiglu_kernel<bf16_t>, grid, dim3(256), 0, stream, (const bf16_t*)x, (bf16_t*)out, I,
+                       grouped);
   else
     return QVL_ERR_DTYPE;
   return qvl_launch_status();

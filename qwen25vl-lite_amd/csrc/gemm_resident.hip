@@ -1,0 +1,242 @@
+// Products with at most 16 rows (a decode step's projections): out[M, N] = X[M, K] . W[N, K]^T,
+// bfloat16 operands, float32 accumulation.  The step is bound by reading W once from HBM, so W
+// is the streamed operand and everything around the product is folded into this kernel, because
+// between two products a short kernel of its own costs more than its arithmetic (its code and
+// data have just been flushed from the caches by the weights).
+//
+// A block of 16 waves owns row tiles of W (16 rows = 16 outputs each; tile, tile + gridDim.x, ...).
+// Wave w covers the 256 values of K from 256 w on, as the A operand (W rows) and B operand (X
+// rows) of v_mfma_f32_16x16x32_bf16; the 16 waves' sums meet in LDS and are added in wave order.
+// If K fits one pass (K <= 4096) the X operand stays in registers for all of the block's tiles and
+// the W loads of the next tile are issued before the current tile's sums are merged; a longer K is
+// walked in passes of 4096.
+//
+// What is folded in:
+//   prologue  PRO_NORM      X = rmsnorm(H) * w, from the float32 residual H (statistics in float32,
+//                           each wave sums its own 256 columns, the block adds the waves in order)
+//   epilogue  EPI_RESIDUAL  out += product, out being the float32 residual
+//             EPI_SWIGLU    W's rows come in groups of 8 gate rows, 8 up rows; out[M, N/2] =
+//                           silu(gate) * up, in bfloat16
+#include "common.h"
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+#define RW 16   // waves per block
+#define RK 8    // 32-wide K steps per wave and pass
+#define PASS_K (RW * RK * 32)
+
+enum { PRO_PLAIN = 0, PRO_NORM = 1 };
+enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2 };
+
+struct ResidentArgs {
+  const bf16_t* X;       // PRO_PLAIN: [M, K]
+  int ldx;
+  const float* H;        // PRO_NORM: float32 [M, K]
+  int ldh;
+  const float* norm_w;   // PRO_NORM: [K]
+  float eps;
+  const bf16_t* W;       // [N, K]
+  int ldw;
+  const float* bias;     // [N] or null (EPI_STORE and EPI_RESIDUAL)
+  void* out;
+  int ldo;
+  int M, N, K, ntiles;
+};
+
+__device__ __forceinline__ bf16x8_t load8(const bf16_t* p) {
+  return __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(p));
+}
+__device__ __forceinline__ bf16x8_t zero8() {
+  u32x4_t z = {0u, 0u, 0u, 0u};
+  return __builtin_bit_cast(bf16x8_t, z);
+}
+__device__ __forceinline__ uint32_t pack2(float a, float b) {
+  bf16x2_t v = {(__bf16)a, (__bf16)b};
+  return __builtin_bit_cast(uint32_t, v);
+}
+
+template <typename TO, int PRO, int EPI, bool ONE_PASS>
+__global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) {
+  __shared__ float red[RW][256];
+  __shared__ float rowsq[RW][16];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lg = lane >> 4, r = lane & 15;
+  const int k_lane = wave * RK * 32 + 8 * lg;  // first K index of this lane within a pass
+  const bool m_ok = r < p.M;
+
+  // ---- the X operand of one pass ------------------------------------------------------------
+  auto load_x = [&](int k0, bf16x8_t* xb) {
+    if (PRO == PRO_PLAIN) {
+      const bf16_t* xrow = p.X + (size_t)(m_ok ? r : 0) * p.ldx;
+#pragma unroll
+      for (int u = 0; u < RK; ++u) {
+        const int k = k0 + k_lane + u * 32;
+        xb[u] = (m_ok && k < p.K) ? load8(xrow + k) : zero8();
+      }
+    } else {
+      // rmsnorm of the float32 rows: this pass covers all of K (ONE_PASS), so the block's waves
+      // hold whole rows between them
+      const float* hrow = p.H + (size_t)(m_ok ? r : 0) * p.ldh;
+      float4 v[RK][2];
+      float ss = 0.f;
+#pragma unroll
+      for (int u = 0; u < RK; ++u) {
+        const int k = k_lane + u * 32;
+        if (m_ok && k < p.K) {
+          v[u][0] = *reinterpret_cast<const float4*>(hrow + k);
+          v[u][1] = *reinterpret_cast<const float4*>(hrow + k + 4);
+        } else {
+          v[u][0] = v[u][1] = float4{0.f, 0.f, 0.f, 0.f};
+        }
+        ss += v[u][0].x * v[u][0].x + v[u][0].y * v[u][0].y + v[u][0].z * v[u][0].z + v[u][0].w * v[u][0].w +
+              v[u][1].x * v[u][1].x + v[u][1].y * v[u][1].y + v[u][1].z * v[u][1].z + v[u][1].w * v[u][1].w;
+      }
+      ss += __shfl_xor(ss, 16, QVL_WAVE);
+      ss += __shfl_xor(ss, 32, QVL_WAVE);
+      if (lg == 0) rowsq[wave][r] = ss;
+      __syncthreads();
+      float total = 0.f;
+#pragma unroll
+      for (int w = 0; w < RW; ++w) total += rowsq[w][r];
+      const float rs = 1.0f / sqrtf(total / (float)p.K + p.eps);
+#pragma unroll
+      for (int u = 0; u < RK; ++u) {
+        const int k = k_lane + u * 32;
+        if (k < p.K) {
+          const float4 g0 = *reinterpret_cast<const float4*>(p.norm_w + k);
+          const float4 g1 = *reinterpret_cast<const float4*>(p.norm_w + k + 4);
+          u32x4_t o = {pack2((v[u][0].x * rs) * g0.x, (v[u][0].y * rs) * g0.y),
+                       pack2((v[u][0].z * rs) * g0.z, (v[u][0].w * rs) * g0.w),
+                       pack2((v[u][1].x * rs) * g1.x, (v[u][1].y * rs) * g1.y),
+                       pack2((v[u][1].z * rs) * g1.z, (v[u][1].w * rs) * g1.w)};
+          xb[u] = __builtin_bit_cast(bf16x8_t, o);
+        } else {
+          xb[u] = zero8();
+        }
+      }
+    }
+  };
+  auto load_w = [&](int tile, int k0, bf16x8_t* a) {
+    const bool row_ok = tile * 16 + r < p.N;
+    const bf16_t* wrow = p.W + (size_t)(row_ok ? tile * 16 + r : 0) * p.ldw;
+#pragma unroll
+    for (int u = 0; u < RK; ++u) {
+      const int k = k0 + k_lane + u * 32;
+      a[u] = (row_ok && k < p.K) ? load8(wrow + k) : zero8();
+    }
+  };
+  // ---- merge the waves' sums of one tile and write the result -----------------------------------
+  auto finish = [&](int tile, const f32x4_t& acc) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) red[wave][(4 * lg + i) * 16 + r] = acc[i];
+    __syncthreads();
+    if (threadIdx.x < 256) {
+      const int e = threadIdx.x;
+      const int m = e >> 4, nl = e & 15, n = tile * 16 + nl;
+      float sum = 0.f;
+#pragma unroll
+      for (int w = 0; w < RW; ++w) sum += red[w][nl * 16 + m];
+      if (EPI == EPI_SWIGLU) {
+        const float up = __shfl_down(sum, 8, QVL_WAVE);  // rows 8..15 of the tile are the up rows
+        if (nl < 8 && m < p.M && n < p.N) {
+          bf16_t* o = reinterpret_cast<bf16_t*>(p.out);
+          o[(size_t)m * p.ldo + tile * 8 + nl] = f32_to_bf16((sum / (1.0f + expf(-sum))) * up);
+        }
+      } else if (m < p.M && n < p.N) {
+        if (p.bias) sum += p.bias[n];
+        if (EPI == EPI_RESIDUAL) {
+          float* o = reinterpret_cast<float*>(p.out);
+          o[(size_t)m * p.ldo + n] += sum;
+        } else {
+          stf<TO>(reinterpret_cast<TO*>(p.out) + (size_t)m * p.ldo + n, sum);
+        }
+      }
+    }
+    __syncthreads();
+  };
+  auto product = [&](const bf16x8_t* a, const bf16x8_t* xb, f32x4_t acc) {
+#pragma unroll
+    for (int u = 0; u < RK; ++u) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], xb[u], acc, 0, 0, 0);
+    return acc;
+  };
+  const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
+
+  if (ONE_PASS) {
+    bf16x8_t xb[RK];
+    bf16x8_t a[2][RK];
+    int tile = blockIdx.x;
+    if (tile < p.ntiles) load_w(tile, 0, a[0]);  // W first: it does not wait for the norm's barrier
+    load_x(0, xb);
+    for (; tile < p.ntiles; tile += 2 * gridDim.x) {
+      const int t1 = tile + gridDim.x, t2 = tile + 2 * gridDim.x;
+      if (t1 < p.ntiles) load_w(t1, 0, a[1]);
+      finish(tile, product(a[0], xb, zero));
+      if (t1 >= p.ntiles) break;
+      if (t2 < p.ntiles) load_w(t2, 0, a[0]);
+      finish(t1, product(a[1], xb, zero));
+    }
+  } else {
+    for (int tile = blockIdx.x; tile < p.ntiles; tile += gridDim.x) {
+      f32x4_t acc = zero;
+      for (int k0 = 0; k0 < p.K; k0 += PASS_K) {
+        bf16x8_t xb[RK], a[RK];
+        load_w(tile, k0, a);
+        load_x(k0, xb);
+        acc = product(a, xb, acc);
+      }
+      finish(tile, acc);
+    }
+  }
+}
+
+template <typename TO, int PRO, int EPI>
+static void launch(const ResidentArgs& p, int blocks, hipStream_t stream) {
+  const dim3 grid(blocks < p.ntiles ? blocks : p.ntiles), block(64 * RW);
+  if (p.K <= PASS_K)
+    hipLaunchKernelGGL((gemm_resident_kernel<TO, PRO, EPI, true>), grid, block, 0, stream, p);
+  else
+    hipLaunchKernelGGL((gemm_resident_kernel<TO, PRO, EPI, false>), grid, block, 0, stream, p);
+}
+
+extern "C" int qvl_gemm_resident_pass_k() { return PASS_K; }
+
+// x: bfloat16 [M, K] (h null), or h: float32 [M, K] with norm_w [K] and eps (x null): X = rmsnorm(h) * norm_w.
+// epilogue 0: out[M, N] in out_dtype (0 float32, 1 bfloat16); 1: out (float32 [M, N]) += product;
+// 2: out[M, N/2] bfloat16 = silu(gate) * up for W rows in groups of 8 gate, 8 up.
+// max_blocks: blocks to launch at most (the number of compute units).
+extern "C" int qvl_gemm_resident(const void* x, int ldx, const void* h, int ldh, const void* norm_w, float eps,
+                                 const void* W, int ldw, const void* bias, void* out, int ldo, int M, int N, int K,
+                                 int out_dtype, int epilogue, int max_blocks, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return QVL_OK;
+  if (M > 16) return QVL_ERR_LIMIT;
+  if (K <= 0 || K % 8 || ldw % 8 || ldw < K || max_blocks <= 0 || !W || !out) return QVL_ERR_SHAPE;
+  const bool norm = h != nullptr;
+  if (norm) {
+    if (x || !norm_w || K > PASS_K || ldh % 4 || ldh < K) return QVL_ERR_SHAPE;
+  } else if (!x || ldx % 8 || ldx < K) {
+    return QVL_ERR_SHAPE;
+  }
+  if (epilogue == EPI_SWIGLU) {
+    if (N % 16 || ldo < N / 2 || bias) return QVL_ERR_SHAPE;
+  } else if (ldo < N) {
+    return QVL_ERR_SHAPE;
+  }
+  ResidentArgs p;
+  p.X = (const bf16_t*)x; p.ldx = ldx; p.H = (const float*)h; p.ldh = ldh; p.norm_w = (const float*)norm_w;
+  p.eps = eps; p.W = (const bf16_t*)W; p.ldw = ldw; p.bias = (const float*)bias; p.out = out; p.ldo = ldo;
+  p.M = M; p.N = N; p.K = K; p.ntiles = (N + 15) / 16;
+#define QVL_RES(TO, EPI)                                                    \
+  do {                                                                      \
+    if (norm) launch<TO, PRO_NORM, EPI>(p, max_blocks, stream);             \
+    else launch<TO, PRO_PLAIN, EPI>(p, max_blocks, stream);                 \
+  } while (0)
+  if (epilogue == EPI_STORE && out_dtype == 0) QVL_RES(float, EPI_STORE);
+  else if (epilogue == EPI_STORE && out_dtype == 1) QVL_RES(bf16_t, EPI_STORE);
+  else if (epilogue == EPI_RESIDUAL) QVL_RES(float, EPI_RESIDUAL);
+  else if (epilogue == EPI_SWIGLU) QVL_RES(bf16_t, EPI_SWIGLU);
+  else return QVL_ERR_DTYPE;
+#undef QVL_RES
+  return qvl_launch_status();
+}

@@ -82,108 +82,6 @@ __global__ __launch_bounds__(64 * NW) void gemm_skinny_kernel(const bf16_t* __re
   }
 }
 
-// ---- M <= 16: the rows of X stay in registers ------------------------------------------------
-// A block of RW waves covers RW * RK * 32 values of K (4096): wave w holds the X operand of its
-// own 256 values of K in registers and walks row tiles of W (tile, tile + gridDim.x, ...) with
-// them, so X is read once per block instead of once per tile, and the loads of the next tile are
-// issued before the waves' sums of the current one meet in LDS.  A longer K is cut into slabs
-// (blockIdx.y); each slab writes its own partial output [slab][M][N], which the consumer adds up
-// in slab order.
-#define RW 16  // waves per block
-#define RK 8   // 32-wide K steps per wave
-
-template <typename TO>
-__global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(const bf16_t* __restrict__ X, int ldx,
-                                                                const bf16_t* __restrict__ W, int ldw,
-                                                                const float* __restrict__ bias, TO* __restrict__ out,
-                                                                int ldo, size_t slab_stride, int M, int N, int K,
-                                                                int ntiles) {
-  __shared__ float red[RW][256];
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lg = lane >> 4, r = lane & 15;
-  const int slab = blockIdx.y;
-  const int k_base = (slab * RW + wave) * RK * 32 + 8 * lg;
-  bf16x8_t xb[RK];
-  {
-    const bool m_ok = r < M;
-    const bf16_t* xrow = X + (size_t)(m_ok ? r : 0) * ldx;
-#pragma unroll
-    for (int u = 0; u < RK; ++u) {
-      const int k = k_base + u * 32;
-      xb[u] = (m_ok && k < K) ? load8(xrow + k) : zero8();
-    }
-  }
-  TO* dst = out + (size_t)slab * slab_stride;
-  const bool add_bias = bias && slab == 0;
-
-  bf16x8_t a[2][RK];
-  int tile = blockIdx.x;
-  auto issue = [&](int t, bf16x8_t* dstregs) {
-    const bool row_ok = t * 16 + r < N;
-    const bf16_t* wrow = W + (size_t)(row_ok ? t * 16 + r : 0) * ldw;
-#pragma unroll
-    for (int u = 0; u < RK; ++u) {
-      const int k = k_base + u * 32;
-      dstregs[u] = (row_ok && k < K) ? load8(wrow + k) : zero8();
-    }
-  };
-  auto finish = [&](int t, const bf16x8_t* regs) {
-    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int u = 0; u < RK; ++u) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(regs[u], xb[u], acc, 0, 0, 0);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) red[wave][(4 * lg + i) * 16 + r] = acc[i];
-    __syncthreads();
-    if (threadIdx.x < 256) {
-      const int e = threadIdx.x;
-      const int m = e >> 4, n = t * 16 + (e & 15);
-      if (m < M && n < N) {
-        float sum = 0.f;
-#pragma unroll
-        for (int w = 0; w < RW; ++w) sum += red[w][(e & 15) * 16 + (e >> 4)];
-        if (add_bias) sum += bias[n];
-        stf<TO>(dst + (size_t)m * ldo + n, sum);
-      }
-    }
-    __syncthreads();
-  };
-  if (tile < ntiles) issue(tile, a[0]);
-  for (; tile < ntiles; tile += 2 * gridDim.x) {
-    const int t1 = tile + gridDim.x, t2 = tile + 2 * gridDim.x;
-    if (t1 < ntiles) issue(t1, a[1]);
-    finish(tile, a[0]);
-    if (t1 >= ntiles) break;
-    if (t2 < ntiles) issue(t2, a[0]);
-    finish(t1, a[1]);
-  }
-}
-
-// Slabs a product with inner size K is written in (1 unless K > 4096).
-extern "C" int qvl_gemm_resident_slabs(int K) { return (K + RW * RK * 32 - 1) / (RW * RK * 32); }
-
-extern "C" int qvl_gemm_resident(const void* X, int ldx, const void* W, int ldw, const void* bias, void* out, int ldo,
-                                 long long slab_stride, int M, int N, int K, int out_dtype, int max_blocks,
-                                 hipStream_t stream) {
-  if (M <= 0 || N <= 0) return QVL_OK;
-  if (M > 16) return QVL_ERR_LIMIT;
-  if (K <= 0 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || ldw < K || ldo < N || max_blocks <= 0) return QVL_ERR_SHAPE;
-  const int slabs = qvl_gemm_resident_slabs(K);
-  if (slabs > 1 && slab_stride < (long long)M * ldo) return QVL_ERR_SHAPE;
-  const int ntiles = (N + 15) / 16;
-  int gx = max_blocks / slabs;
-  gx = gx < 1 ? 1 : (gx > ntiles ? ntiles : gx);
-  const dim3 grid(gx, slabs), block(64 * RW);
-  if (out_dtype == 0)
-    hipLaunchKernelGGL(gemm_resident_kernel<float>, grid, block, 0, stream, (const bf16_t*)X, ldx, (const bf16_t*)W,
-                       ldw, (const float*)bias, (float*)out, ldo, (size_t)slab_stride, M, N, K, ntiles);
-  else if (out_dtype == 1 && slabs == 1)
-    hipLaunchKernelGGL(gemm_resident_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)X, ldx,
-                       (const bf16_t*)W, ldw, (const float*)bias, (bf16_t*)out, ldo, (size_t)slab_stride, M, N, K,
-                       ntiles);
-  else
-    return QVL_ERR_DTYPE;  // partial sums are float32
-  return qvl_launch_status();
-}
-
 template <typename TO>
 static int launch(const void* X, int ldx, const void* W, int ldw, const void* bias, void* out, int ldo, int M, int N,
                   int K, hipStream_t stream) {

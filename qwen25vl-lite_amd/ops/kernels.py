@@ -94,8 +94,6 @@ def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Te
                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``h += delta`` (float32 sum) and return ``rmsnorm(h) * weight`` in ``out_dtype``.
 
-    ``delta`` may be ``[S, N, H]``: partial sums of a product, added in slab order.
-
     With ``rows`` (int32 row indices) only those rows are normalised and ``h`` is not written.
     """
     _dev(h, delta, weight, rows, out)
@@ -103,12 +101,8 @@ def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Te
     n, width = h.shape
     _need(weight.dtype == torch.float32 and weight.shape == (width,) and weight.is_contiguous(),
           "norm weight must be float32 [H]")
-    slabs, slab_stride = 1, 0
     if delta is not None:
-        _need(delta.is_contiguous() and tuple(delta.shape[-2:]) == tuple(h.shape) and delta.dim() in (2, 3),
-              "delta must be [N, H] or slabs [S, N, H]")
-        if delta.dim() == 3:
-            slabs, slab_stride = delta.shape[0], delta.stride(0)
+        _need(delta.shape == h.shape and delta.is_contiguous(), "delta must match h's shape")
     m = n
     if rows is not None:
         _need(rows.dtype == torch.int32 and rows.dim() == 1 and rows.is_contiguous(), "rows must be int32 [M]")
@@ -117,11 +111,10 @@ def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Te
         out = torch.empty((m, width), dtype=out_dtype, device=h.device)
     _need(out.shape == (m, width) and out.dtype == out_dtype and out.is_contiguous(), "out must be [M, H]")
     fn = _fn("elementwise", "qvl_add_rmsnorm",
-             [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int,
-              ctypes.c_longlong, _c_ptr])
+             [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr])
     _check(fn(_ptr(h), _ptr(delta), _ptr(weight), _ptr(out), _ptr(rows), m, width, float(eps),
-              dtype_code(delta.dtype if delta is not None else out_dtype), dtype_code(out_dtype), slabs, slab_stride,
-              _stream()), "add_rmsnorm")
+              dtype_code(delta.dtype if delta is not None else out_dtype), dtype_code(out_dtype), _stream()),
+           "add_rmsnorm")
     return out
 
 
@@ -210,16 +203,18 @@ def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     return out
 
 
-def swiglu(x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """``silu(x[:, :I]) * x[:, I:]`` for ``x`` of ``[N, 2 I]``."""
+def swiglu(x: torch.Tensor, out: Optional[torch.Tensor] = None, grouped: bool = False) -> torch.Tensor:
+    """``silu(gate) * up`` for ``x`` of ``[N, 2 I]``: gate in the first ``I`` columns and up in the
+    rest, or, ``grouped``, in alternating groups of 8 gate and 8 up columns."""
     _dev(x, out)
     _need(x.dim() == 2 and x.shape[1] % 2 == 0 and x.is_contiguous(), "x must be contiguous [N, 2 I]")
     n, inter = x.shape[0], x.shape[1] // 2
     if out is None:
         out = torch.empty((n, inter), dtype=x.dtype, device=x.device)
     _need(out.shape == (n, inter) and out.dtype == x.dtype and out.is_contiguous(), "out must be [N, I]")
-    fn = _fn("elementwise", "qvl_swiglu", [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr])
-    _check(fn(_ptr(x), _ptr(out), n, inter, dtype_code(x.dtype), _stream()), "swiglu")
+    _need(not grouped or inter % 8 == 0, "grouped columns need a width in steps of 8")
+    fn = _fn("elementwise", "qvl_swiglu", [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(x), _ptr(out), n, inter, dtype_code(x.dtype), int(grouped), _stream()), "swiglu")
     return out
 
 

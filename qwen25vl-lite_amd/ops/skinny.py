@@ -1,4 +1,9 @@
-"""Dispatch of bfloat16 products with few rows to the hand-written skinny kernel."""
+"""Dispatch of bfloat16 products with few rows to the hand-written kernels.
+
+Up to 16 rows: the resident kernel (``csrc/gemm_resident.hip``), which can also fold the RMSNorm
+before the product, the residual add after it, or the SwiGLU activation into itself.
+17 to 32 rows: the streaming kernel (``csrc/gemm_skinny.hip``) where it beats the library.
+"""
 
 from __future__ import annotations
 
@@ -9,30 +14,14 @@ import torch
 
 from .kernels import _check, _fn, _ptr, _stream, dtype_code
 
-__all__ = ["try_linear", "MAX_ROWS"]
+__all__ = ["resident_product", "takes_resident", "try_streaming", "RESIDENT_ROWS", "RESIDENT_NORM_K", "MAX_ROWS",
+           "STORE", "RESIDUAL", "SWIGLU"]
 
-MAX_ROWS = 64
-_c_int, _c_ptr = ctypes.c_int, ctypes.c_void_p
-
-
-def prefers_skinny(m: int, n: int, k: int) -> bool:
-    """Where the streaming skinny kernel (rows of x read again from L2 by every wave) beats the
-    library's product on MI355X, measured at the 7B decoder's shapes: always up to 4 rows; with
-    more rows the rows of x weigh more, and the library wins on the large matrices."""
-    size = n * k
-    if m <= 4:
-        return True
-    if m <= 8:
-        return size <= 72_000_000
-    if m <= 16:
-        return size <= 20_000_000
-    if m <= 32:
-        return size <= 13_000_000 or k >= 4 * n
-    return False
-
-
-RESIDENT_ROWS = 16       # up to here the rows of x stay in registers
-RESIDENT_K = 4096        # inner size one block of the resident kernel covers
+MAX_ROWS = 32            # the streaming kernel's limit in use
+RESIDENT_ROWS = 16       # up to here the resident kernel runs
+RESIDENT_NORM_K = 4096   # the folded norm needs the whole row in one pass of the block
+STORE, RESIDUAL, SWIGLU = 0, 1, 2
+_c_int, _c_float, _c_ptr = ctypes.c_int, ctypes.c_float, ctypes.c_void_p
 _cu_count = {}
 
 
@@ -43,36 +32,71 @@ def _compute_units(device) -> int:
     return _cu_count[key]
 
 
-def try_linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
-               out_dtype: Optional[torch.dtype], allow_slabs: bool = False) -> Optional[torch.Tensor]:
-    """``x @ weight.T (+ bias)`` through a skinny kernel, or None if the shape is not one they take
-    (too many rows, an inner size that is not a multiple of 8, rows that are not 16-byte aligned).
+def _rows_aligned(t: torch.Tensor, elems: int) -> bool:
+    return t.stride(1) == 1 and t.stride(0) % elems == 0 and t.data_ptr() % 16 == 0
 
-    Up to 16 rows the resident kernel runs.  An inner size above 4096 makes it write partial sums
-    in slabs ``[S, M, N]`` (float32), which the caller must have asked for with ``allow_slabs`` and
-    whose consumer adds them up in slab order (the residual add + norm kernel does)."""
+
+def takes_resident(m: int, k: int, weight: torch.Tensor, *, norm: bool = False) -> bool:
+    """Whether the resident kernel takes a product of ``m`` rows with this weight."""
+    if m > RESIDENT_ROWS or k % 8 or weight.dtype != torch.bfloat16 or not _rows_aligned(weight, 8):
+        return False
+    return not norm or k <= RESIDENT_NORM_K
+
+
+def resident_product(weight: torch.Tensor, *, x: Optional[torch.Tensor] = None, h: Optional[torch.Tensor] = None,
+                     norm_weight: Optional[torch.Tensor] = None, eps: float = 0.0,
+                     bias: Optional[torch.Tensor] = None, epilogue: int = STORE,
+                     out: Optional[torch.Tensor] = None, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """``X @ weight.T`` for at most 16 rows.  ``X`` is ``x`` (bfloat16), or ``rmsnorm(h) * norm_weight``
+    formed inside the kernel from the float32 rows ``h``.  ``epilogue``: ``STORE`` writes the product
+    (plus ``bias``) to a new tensor of ``out_dtype``; ``RESIDUAL`` adds it to ``out`` (float32) in
+    place; ``SWIGLU`` takes ``weight``'s rows as groups of 8 gate, 8 up rows and returns
+    ``silu(gate) * up`` as bfloat16 ``[M, N/2]``."""
+    src = x if x is not None else h
+    m, k = src.shape
+    n = weight.shape[0]
+    if not takes_resident(m, k, weight, norm=h is not None) or weight.shape[1] != k:
+        raise ValueError("the resident kernel does not take this product")
+    if x is not None and (x.dtype != torch.bfloat16 or not _rows_aligned(x, 8)):
+        raise ValueError("x must be bfloat16 with 16-byte aligned rows")
+    if h is not None and (h.dtype != torch.float32 or not _rows_aligned(h, 4) or norm_weight is None
+                          or norm_weight.dtype != torch.float32 or norm_weight.shape != (k,)):
+        raise ValueError("h must be float32 rows with a float32 norm weight of their width")
+    if bias is not None and (bias.dtype != torch.float32 or not bias.is_contiguous() or bias.shape != (n,)):
+        raise ValueError("bias must be float32 [N]")
+    if epilogue == RESIDUAL:
+        if out is None or out.dtype != torch.float32 or out.shape != (m, n) or out.stride(1) != 1:
+            raise ValueError("the residual must be float32 [M, N]")
+        odt = torch.float32
+    elif epilogue == SWIGLU:
+        if n % 16:
+            raise ValueError("gate | up rows must come in groups of 8 + 8")
+        out, odt = torch.empty((m, n // 2), dtype=torch.bfloat16, device=src.device), torch.bfloat16
+    else:
+        out, odt = torch.empty((m, n), dtype=out_dtype, device=src.device), out_dtype
+    fn = _fn("gemm_resident", "qvl_gemm_resident",
+             [_c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_float, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int,
+              _c_int, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(x), x.stride(0) if x is not None else 0, _ptr(h), h.stride(0) if h is not None else 0,
+              _ptr(norm_weight), float(eps), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(out), out.stride(0),
+              m, n, k, dtype_code(odt), epilogue, _compute_units(src.device), _stream()), "linear (resident)")
+    return out
+
+
+def prefers_streaming(m: int, n: int, k: int) -> bool:
+    """Where the streaming kernel (rows of x read again from L2 by every wave) beats the library's
+    product on MI355X, measured at the 7B decoder's shapes with 17 to 32 rows: the small square
+    matrix and the one with a long inner size."""
+    return RESIDENT_ROWS < m <= MAX_ROWS and (n * k <= 13_000_000 or k >= 4 * n)
+
+
+def try_streaming(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
+                  out_dtype: Optional[torch.dtype]) -> Optional[torch.Tensor]:
+    """``x @ weight.T (+ bias)`` through the streaming kernel, or None if it is not the better choice
+    or does not take the shape."""
     m, k = x.shape
     n = weight.shape[0]
-    aligned = (k % 8 == 0 and x.stride(1) == 1 and weight.stride(1) == 1 and x.stride(0) % 8 == 0
-               and weight.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
-    bias_ok = bias is None or (bias.dtype == torch.float32 and bias.is_contiguous() and bias.shape == (n,))
-    odt = out_dtype or x.dtype
-    slabs = (k + RESIDENT_K - 1) // RESIDENT_K
-    if (m <= RESIDENT_ROWS and aligned and bias_ok
-            and (slabs == 1 or (allow_slabs and odt == torch.float32))):
-        shape = (m, n) if slabs == 1 else (slabs, m, n)
-        out = torch.empty(shape, dtype=odt, device=x.device)
-        fn = _fn("gemm_skinny", "qvl_gemm_resident",
-                 [_c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, ctypes.c_longlong, _c_int, _c_int, _c_int,
-                  _c_int, _c_int, _c_ptr])
-        _check(fn(_ptr(x), x.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(out), n, m * n, m, n, k,
-                  dtype_code(odt), _compute_units(x.device), _stream()), "linear (skinny, resident)")
-        return out
-    if not prefers_skinny(m, n, k):
-        return None
-    if m > MAX_ROWS or k % 8 or x.stride(1) != 1 or weight.stride(1) != 1 or x.stride(0) % 8 or weight.stride(0) % 8:
-        return None
-    if x.data_ptr() % 16 or weight.data_ptr() % 16:
+    if not prefers_streaming(m, n, k) or k % 8 or not _rows_aligned(x, 8) or not _rows_aligned(weight, 8):
         return None
     if bias is not None and (bias.dtype != torch.float32 or not bias.is_contiguous() or bias.shape != (n,)):
         return None
@@ -81,5 +105,5 @@ def try_linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tenso
     fn = _fn("gemm_skinny", "qvl_gemm_skinny",
              [_c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
     _check(fn(_ptr(x), x.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(out), out.stride(0), m, n, k,
-              dtype_code(odt), _stream()), "linear (skinny)")
+              dtype_code(odt), _stream()), "linear (streaming)")
     return out

@@ -14,7 +14,7 @@ import torch
 
 from ..ops import kernels
 from ..ops.attention import paged_attention
-from ..ops.linear import linear
+from ..ops.linear import linear, linear_into
 from .base import (CacheNeed, LayerSlot, Mixer, ParamSpec, PartSpec, StepContext, build_part, register_part)
 
 __all__ = ["PagedAttention"]
@@ -27,6 +27,7 @@ class PagedAttention(Mixer):
     has no key/value projections and reads the cache another layer wrote)."""
 
     graph_safe = True
+    takes_lazy_norm = True
 
     def __init__(self, params, dtype, device):
         super().__init__(dtype, device)
@@ -101,7 +102,7 @@ class PagedAttention(Mixer):
             group.slot_mapping if write else None, slot.k_cache if write else None, slot.v_cache if write else None,
             self.nq, self.nkv if write else 0, self.hd, group.page_size, out_dtype=self.dtype)
         o = paged_attention(q, slot.k_cache, slot.v_cache, group.block_table, step, self.nq, self.window, self.scale)
-        return linear(o, self.w_out, out_dtype=torch.float32, allow_slabs=True)
+        return linear_into(step.residual, o, self.w_out)
 
 
 register_part("mixer", "paged_attention", PagedAttention)

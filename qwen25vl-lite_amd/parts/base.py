@@ -8,11 +8,14 @@ Kinds of parts and what each must provide:
 
 * ``Norm``: ``forward(stream) -> x``.  Folds the stream's pending addend into the float32
   residual and returns the normalised activations in the run dtype.
-* ``Mixer``: ``forward(x, step, slot) -> y`` for ``x`` of ``[N, hidden]`` (``y`` may also be
-  partial sums ``[S, N, hidden]``, which the next norm adds up); it may keep keys and
+* ``Mixer``: ``forward(x, step, slot) -> y`` for ``x`` of ``[N, hidden]``; it may keep keys and
   values in pages (``cache_need()``) and/or a state of fixed size per request
   (``state_need()``), both handed to it through ``slot``.
 * ``FeedForward``: ``forward(x, step) -> y``.
+  A mixer or feed-forward may add ``y`` into ``step.residual`` (the float32 residual, if the block
+  offers it) itself and return None; one that sets ``takes_lazy_norm`` may be handed
+  :class:`~qwen25vl_lite_amd.ops.linear.NormedRows` instead of a tensor and passes it to its first
+  product, which then computes the norm on the way.
 * ``PositionEncoding``: ``rotary_tables(head_dim, device)`` gives the per-frequency inverse
   frequencies and the row of the position tensor each frequency reads.
 * ``Block``: ``forward(stream, step, slot)`` arranges two norms, a mixer and a feed-forward.
@@ -113,6 +116,7 @@ class StepContext:
     max_q_len: int = 0
     max_ctx_len: int = 0
     dtype: torch.dtype = torch.float32
+    residual: Optional[torch.Tensor] = None   # set by a block while a part may add its result in place
     derived: Dict[Any, Any] = field(default_factory=dict)   # per-step arrays kernels derive once (tile lists)
 
 
@@ -122,7 +126,7 @@ class ResidualStream:
     norm adds ``pending`` to ``h`` in float32 in the same kernel that normalises."""
 
     h: torch.Tensor                          # float32 [N, hidden]
-    pending: Optional[torch.Tensor] = None   # [N, hidden], or partial sums [S, N, hidden] added in order
+    pending: Optional[torch.Tensor] = None   # float32 or run dtype [N, hidden]
 
 
 class Part:
@@ -131,6 +135,7 @@ class Part:
     the step's values), so a decode step through it may be captured in a HIP graph."""
 
     graph_safe: bool = False
+    takes_lazy_norm: bool = False   # forward accepts NormedRows in place of the normalised tensor
 
     def __init__(self, dtype: torch.dtype, device: torch.device):
         self.dtype = dtype
@@ -147,7 +152,9 @@ class Part:
 
 
 class Norm(Part):
-    def forward(self, stream: ResidualStream, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    def forward(self, stream: ResidualStream, rows: Optional[torch.Tensor] = None, lazy: bool = False):
+        """Fold ``stream.pending`` into ``stream.h`` and return the normalised rows; with ``lazy`` it
+        may return :class:`~qwen25vl_lite_amd.ops.linear.NormedRows` instead of computing them."""
         raise NotImplementedError
 
 

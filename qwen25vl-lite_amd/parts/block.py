@@ -13,8 +13,9 @@ class PreNormBlock(Block):
     """``h += mixer(norm1(h)); h += ffn(norm2(h))``.
 
     params: ``norm1``, ``mixer``, ``norm2``, ``ffn`` (:class:`PartSpec` each) and ``names``,
-    the checkpoint sub-name of each of the four.  Each sum into ``h`` happens in float32
-    inside the following norm's kernel (the last one in the model's final norm).
+    the checkpoint sub-name of each of the four.  Each sum into ``h`` happens in float32,
+    inside the following norm's kernel or, in a decode step, inside the product that ends the
+    mixer or the feed-forward.
     """
 
     graph_safe = True
@@ -32,10 +33,13 @@ class PreNormBlock(Block):
                 self.names["norm2"]: self.norm2, self.names["ffn"]: self.ffn}
 
     def forward(self, stream: ResidualStream, step: StepContext, slot: LayerSlot) -> ResidualStream:
-        x = self.norm1.forward(stream)
+        x = self.norm1.forward(stream, lazy=self.mixer.takes_lazy_norm)
+        step.residual = stream.h            # the mixer may add its result in place and return None
         stream.pending = self.mixer.forward(x, step, slot)
-        y = self.norm2.forward(stream)
+        y = self.norm2.forward(stream, lazy=self.ffn.takes_lazy_norm)
+        step.residual = stream.h
         stream.pending = self.ffn.forward(y, step)
+        step.residual = None
         return stream
 
 

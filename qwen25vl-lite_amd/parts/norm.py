@@ -6,7 +6,8 @@ from typing import Dict, Optional
 
 import torch
 
-from ..ops import kernels
+from ..ops import kernels, skinny
+from ..ops.linear import NormedRows
 from .base import Norm, ParamSpec, ResidualStream, register_part
 
 __all__ = ["RMSNorm"]
@@ -33,7 +34,12 @@ class RMSNorm(Norm):
     def load(self, tensors):
         self.weight = tensors["weight"]
 
-    def forward(self, stream: ResidualStream, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    def forward(self, stream: ResidualStream, rows: Optional[torch.Tensor] = None, lazy: bool = False):
+        if (lazy and rows is None and stream.pending is None and self.dtype == torch.bfloat16
+                and stream.h.shape[0] <= skinny.RESIDENT_ROWS and self.size % 8 == 0
+                and self.size <= skinny.RESIDENT_NORM_K):
+            # a decode step: the product that follows computes the norm on the way
+            return NormedRows(stream.h, self.weight, self.eps, self.dtype)
         out = kernels.add_rmsnorm(stream.h, stream.pending, self.weight, self.eps, self.dtype, rows=rows)
         if rows is None:
             stream.pending = None  # folded into h

@@ -43,12 +43,6 @@ def test_add_rmsnorm(width, delta_dtype, out_dtype):
     assert out.dtype == out_dtype
     assert torch.allclose(out.float().cpu(), want, **_tol(out_dtype))
     assert torch.allclose(hd.cpu(), total, atol=1e-6), "the sum is written back in float32"
-    if delta is not None and delta_dtype == torch.float32:
-        # partial sums in slabs are added in order
-        parts = torch.stack([delta * 0.25, delta * 0.5, delta * 0.25])
-        hd = h.cuda()
-        out = kernels.add_rmsnorm(hd, parts.cuda(), w.cuda(), eps, out_dtype)
-        assert torch.allclose(out.float().cpu(), want, **_tol(out_dtype)) and torch.allclose(hd.cpu(), total, atol=1e-5)
     # selected rows: h stays as it was
     hd = h.cuda()
     rows = torch.tensor([4, 0, 4], dtype=torch.int32).cuda()
@@ -202,6 +196,10 @@ def test_swiglu(dtype, rows, inter):
     want = torch.nn.functional.silu(x[:, :inter].float()) * x[:, inter:].float()
     out = kernels.swiglu(x.cuda())
     assert torch.allclose(out.float().cpu(), want, **_tol(dtype))
+    if inter % 8 == 0:   # the same values with gate and up columns in alternating groups of 8
+        g = torch.stack([x[:, :inter].reshape(rows, -1, 8), x[:, inter:].reshape(rows, -1, 8)], dim=2)
+        out = kernels.swiglu(g.reshape(rows, 2 * inter).contiguous().cuda(), grouped=True)
+        assert torch.allclose(out.float().cpu(), want, **_tol(dtype))
 
 
 @pytest.mark.parametrize("m, n, k", [(1, 5, 3), (7, 509, 144), (65, 130, 353), (130, 64, 1000)])
@@ -221,25 +219,19 @@ def test_gemm_f32_is_exact_and_row_independent(m, n, k):
     assert torch.equal(alone[0], out[m // 2])
 
 
-@pytest.mark.parametrize("m, n, k", [(1, 509, 144), (8, 300, 200), (16, 17, 8), (9, 100, 8200), (17, 1000, 4104), (31, 130, 352),
-                                     (64, 509, 3584), (5, 40, 100), (300, 64, 1000)])
+@pytest.mark.parametrize("m, n, k", [(1, 509, 144), (8, 300, 200), (16, 17, 8), (9, 100, 8200), (17, 1000, 4104),
+                                     (31, 130, 352), (64, 509, 3584), (5, 40, 100), (300, 64, 1000)])
 def test_linear_bfloat16(m, n, k):
-    """Few rows go through the skinny matrix-core kernel (inner sizes in steps of 8), the rest
-    through the library; both accumulate in float32."""
+    """Up to 16 rows go through the resident matrix-core kernel (inner sizes in steps of 8, any
+    length), 17 to 32 through the streaming one where it wins, the rest through the library; all
+    accumulate in float32."""
     from qwen25vl_lite_amd.ops import skinny
     from qwen25vl_lite_amd.ops.linear import linear
     torch.manual_seed(k)
     x, w = torch.randn(m, k).bfloat16(), (torch.randn(n, k) / math.sqrt(k)).bfloat16()
     b = torch.randn(n)
     want = x.float() @ w.float().T
-    took = skinny.try_linear(x.cuda(), w.cuda(), None, torch.float32)
-    assert (took is not None) == (m <= 32 and k % 8 == 0)
-    if m <= 16 and k % 8 == 0:
-        # an inner size above 4096 comes as partial sums in slabs, if the caller takes them
-        slabs = skinny.try_linear(x.cuda(), w.cuda(), None, torch.float32, allow_slabs=True)
-        assert slabs.dim() == (3 if k > 4096 else 2)
-        total = slabs.sum(0) if slabs.dim() == 3 else slabs
-        assert torch.allclose(total.cpu(), want, atol=2e-3, rtol=2e-3)
+    assert skinny.takes_resident(m, k, w.cuda()) == (m <= 16 and k % 8 == 0)
     out32 = linear(x.cuda(), w.cuda(), out_dtype=torch.float32)
     assert out32.dtype == torch.float32 and torch.allclose(out32.cpu(), want, atol=2e-3, rtol=2e-3)
     out16 = linear(x.cuda(), w.cuda())
@@ -250,6 +242,64 @@ def test_linear_bfloat16(m, n, k):
     if m > 1:
         alone = linear(x[m // 2:m // 2 + 1].contiguous().cuda(), w.cuda(), out_dtype=torch.float32)
         assert torch.allclose(alone[0], out32[m // 2], atol=1e-5, rtol=1e-5)
+
+
+@pytest.mark.parametrize("m, n, k", [(1, 48, 64), (7, 1000, 3584), (16, 130, 4096), (3, 64, 144)])
+def test_product_with_the_norm_folded_in(m, n, k):
+    """rmsnorm(h) * w formed inside the product equals the norm kernel followed by the product."""
+    from qwen25vl_lite_amd.ops import kernels
+    from qwen25vl_lite_amd.ops.linear import NormedRows, linear
+    torch.manual_seed(n)
+    h = (torch.randn(m, k) * 2).cuda()
+    g = (1 + 0.1 * torch.randn(k)).cuda()
+    w = (torch.randn(n, k) / math.sqrt(k)).bfloat16().cuda()
+    fused = linear(NormedRows(h, g, 1e-5, torch.bfloat16), w, out_dtype=torch.float32)
+    apart = linear(kernels.add_rmsnorm(h, None, g, 1e-5, torch.bfloat16), w, out_dtype=torch.float32)
+    want = plain_rmsnorm(h.cpu(), g.cpu(), 1e-5).bfloat16().float() @ w.float().cpu().T
+    assert torch.allclose(fused.cpu(), want, atol=3e-3, rtol=3e-3)
+    assert (fused - apart).abs().max() < 0.02 * want.abs().max()   # the same up to a bfloat16 rounding of x here and there
+    # a longer row than one pass of the block holds is computed by the norm's own kernel first
+    h2, g2 = torch.randn(2, 4104).cuda(), torch.ones(4104).cuda()
+    w2 = (torch.randn(24, 4104) / 64).bfloat16().cuda()
+    out = linear(NormedRows(h2, g2, 1e-6, torch.bfloat16), w2, out_dtype=torch.float32)
+    assert torch.allclose(out.cpu(), plain_rmsnorm(h2.cpu(), g2.cpu(), 1e-6).bfloat16().float() @ w2.float().cpu().T,
+                          atol=3e-3, rtol=3e-3)
+
+
+@pytest.mark.parametrize("m, n, k", [(1, 144, 352), (8, 3584, 18944), (16, 100, 4104), (40, 144, 352)])
+def test_product_added_into_the_residual(m, n, k):
+    from qwen25vl_lite_amd.ops.linear import linear_into
+    torch.manual_seed(k)
+    x = torch.randn(m, k).bfloat16().cuda()
+    w = (torch.randn(n, k) / math.sqrt(k)).bfloat16().cuda()
+    h = torch.randn(m, n).cuda()
+    want = h.cpu() + x.float().cpu() @ w.float().cpu().T
+    left = linear_into(h, x, w)
+    if m <= 16:
+        assert left is None and torch.allclose(h.cpu(), want, atol=3e-3, rtol=3e-3)
+    else:   # too many rows for the fused kernel: the product comes back for the next norm to add
+        assert left is not None and left.dtype == torch.float32
+        assert torch.allclose(h.cpu() + left.cpu(), want, atol=3e-3, rtol=3e-3)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m, inter, k", [(1, 352, 144), (8, 18944, 3584), (16, 40, 4104), (50, 352, 144)])
+def test_gate_up_product_with_the_activation_folded_in(dtype, m, inter, k):
+    """Grouped gate | up rows: few bfloat16 rows get silu(gate) * up from the product's own kernel,
+    everything else from the product followed by the activation kernel on the grouped columns."""
+    from qwen25vl_lite_amd.ops.linear import gate_up_swiglu
+    torch.manual_seed(inter)
+    x = torch.randn(m, k).to(dtype)
+    gate = (torch.randn(inter, k) / math.sqrt(k)).to(dtype)
+    up = (torch.randn(inter, k) / math.sqrt(k)).to(dtype)
+    grouped = torch.stack([gate.view(-1, 8, k), up.view(-1, 8, k)], dim=1).reshape(2 * inter, k).contiguous()
+    out = gate_up_swiglu(x.cuda(), grouped.cuda(), True)
+    want = torch.nn.functional.silu(x.float() @ gate.float().T) * (x.float() @ up.float().T)
+    assert out.shape == (m, inter) and out.dtype == dtype
+    tol = dict(atol=1e-4, rtol=1e-4) if dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)
+    assert torch.allclose(out.float().cpu(), want, **tol)
+    plain = gate_up_swiglu(x.cuda(), torch.cat([gate, up]).cuda(), False)
+    assert torch.allclose(plain.float().cpu(), want, **tol)
 
 
 def test_no_cpu_path():
