@@ -95,4 +95,5 @@ def qwen25vl_text_spec(config: Qwen25VLConfig) -> ModelSpec:
 
 
 register_architecture("Qwen2_5_VLForConditionalGeneration", qwen25vl_text_spec)
-register_architecture("qwen2_5_vl", qwen25vl_text_spec)
+register_architecture("qwen2_5_vl", qwen25vl_text_spec)        # model_type, for a config.json without architectures
+register_architecture("qwen2_5_vl_text", qwen25vl_text_spec)   # model_type of a bare text_config
