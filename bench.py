@@ -73,6 +73,7 @@ def main(argv=None) -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and the prefill")
     ap.add_argument("--no-graph", action="store_true", help="do not replay decode steps from a HIP graph")
+    ap.add_argument("--no-tune", action="store_true", help="do not let TunableOp choose the library's kernels")
     args = ap.parse_args(argv)
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print(f"bench.py measures one GPU: this engine does not run on {args.gpus} GPUs (run with --gpus 1)")
@@ -98,7 +99,8 @@ def main(argv=None) -> int:
     def make_engine(max_seqs, tokens_per_seq, budget):
         ecfg = EngineConfig(num_blocks=max_seqs * ((tokens_per_seq + page - 1) // page + 1), block_size=page,
                             max_num_seqs=max_seqs, max_num_batched_tokens=budget, max_model_len=max_ctx,
-                            enable_prefix_cache=False, dtype=dtype, device="cuda:0", hip_graph=not args.no_graph)
+                            enable_prefix_cache=False, dtype=dtype, device="cuda:0", hip_graph=not args.no_graph,
+                            tune_library_products=not args.no_tune)
         runner = ModelRunner(model, ecfg)
         return LLMEngine(runner, ecfg), runner
 
@@ -164,7 +166,7 @@ def main(argv=None) -> int:
             "kv_heads": t.num_key_value_heads, "head_dim": t.head_dim, "intermediate_size": t.intermediate_size,
             "vocab_size": t.vocab_size, "global_batch": args.batch, "seq_len": args.prompt_tokens,
             "context_mid": ctx_mid, "max_context": max_ctx, "page_size": page, "parallelism": "single GPU",
-            "hip_graph": not args.no_graph,
+            "hip_graph": not args.no_graph, "tuned_library_products": not args.no_tune,
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},

@@ -35,7 +35,9 @@ class EngineConfig:
     ``max_num_batched_tokens`` tokens, decoded tokens included; ``max_model_len`` bounds a
     request's prompt plus output.  ``preemption`` is what happens when pages run out:
     only ``"recompute"`` is built (the victim gives its pages back and is prefilled again,
-    prompt and tokens generated so far).
+    prompt and tokens generated so far).  ``hip_graph`` replays decode steps from captured HIP graphs.
+    ``tune_library_products`` lets PyTorch's TunableOp choose the library kernel of each product shape
+    (seconds per new shape, once): for runs with few distinct step sizes.
     """
 
     num_blocks: int = 2048
@@ -49,6 +51,7 @@ class EngineConfig:
     device: str = "cuda:0"
     dtype: torch.dtype = torch.float32
     hip_graph: bool = False
+    tune_library_products: bool = False
 
     def __post_init__(self) -> None:
         self.dtype = dtype_from_name(self.dtype)

@@ -48,6 +48,9 @@ class ModelRunner:
         self.slots = model.make_slots(self.storage, self.states)
         self.position_rows = model.spec.position_rows
         self.steps = 0
+        if engine_cfg.tune_library_products:
+            from ..ops.linear import tune_library_products
+            tune_library_products(True)
         # decode steps from HIP graphs, if asked for and every part can be captured
         self.graphs = None
         if engine_cfg.hip_graph and model.graph_safe:

@@ -15,7 +15,7 @@ import torch
 
 from . import kernels, skinny
 
-__all__ = ["NormedRows", "linear", "linear_into", "gate_up_swiglu"]
+__all__ = ["NormedRows", "linear", "linear_into", "gate_up_swiglu", "tune_library_products"]
 
 
 class NormedRows:
@@ -79,7 +79,26 @@ def linear_into(residual: Optional[torch.Tensor], x: torch.Tensor, weight: torch
             and x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0):
         skinny.resident_product(weight, x=x, epilogue=skinny.RESIDUAL, out=residual)
         return None
-    return linear(x, weight, out_dtype=torch.float32)
+    # More rows: the library's product.  Its bfloat16 output is the form it is tuned for (and the
+    # only one the tuner of `tune_library_products` covers); the sum into the residual stays float32.
+    return linear(x, weight, out_dtype=torch.float32 if x.shape[0] <= skinny.MAX_ROWS else None)
+
+
+def tune_library_products(enable: bool = True, max_ms: int = 3000) -> None:
+    """Let PyTorch's TunableOp pick the fastest library kernel for every product shape it meets
+    (each new shape costs a few seconds once; its choices are kept in a per-user file under the
+    temporary directory).  Meant for runs with few distinct shapes, such as a benchmark; off by
+    default."""
+    import os
+    import tempfile
+
+    import torch.cuda.tunable as tunable
+
+    if enable:
+        tunable.set_filename(os.path.join(tempfile.gettempdir(), f"qwen25vl_lite_amd-tunableop-{os.getuid()}.csv"))
+        tunable.set_max_tuning_duration(int(max_ms))
+    tunable.enable(enable)
+    tunable.tuning_enable(enable)
 
 
 def gate_up_swiglu(x: Union[torch.Tensor, NormedRows], weight: torch.Tensor, grouped: bool) -> torch.Tensor:
