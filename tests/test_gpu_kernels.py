@@ -266,7 +266,7 @@ def test_product_with_the_norm_folded_in(m, n, k):
                           atol=3e-3, rtol=3e-3)
 
 
-@pytest.mark.parametrize("m, n, k", [(1, 144, 352), (8, 3584, 18944), (16, 100, 4104), (40, 144, 352)])
+@pytest.mark.parametrize("m, n, k", [(1, 144, 352), (8, 3584, 18944), (16, 100, 4104), (24, 144, 352), (40, 144, 352)])
 def test_product_added_into_the_residual(m, n, k):
     from qwen25vl_lite_amd.ops.linear import linear_into
     torch.manual_seed(k)
@@ -277,9 +277,11 @@ def test_product_added_into_the_residual(m, n, k):
     left = linear_into(h, x, w)
     if m <= 16:
         assert left is None and torch.allclose(h.cpu(), want, atol=3e-3, rtol=3e-3)
-    else:   # too many rows for the fused kernel: the product comes back for the next norm to add
-        assert left is not None and left.dtype == torch.float32
-        assert torch.allclose(h.cpu() + left.cpu(), want, atol=3e-3, rtol=3e-3)
+    else:   # too many rows for the fused kernel: the product comes back for the next norm to add,
+        # in float32 from the hand-written kernels and in bfloat16 from the library (above 32 rows)
+        assert left is not None and left.dtype == (torch.float32 if m <= 32 else torch.bfloat16)
+        tol = 3e-3 if m <= 32 else 2e-2
+        assert torch.allclose(h.cpu() + left.float().cpu(), want, atol=tol, rtol=tol)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
