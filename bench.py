@@ -72,6 +72,7 @@ def main(argv=None) -> int:
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration has")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and the prefill")
+    ap.add_argument("--prefill-only", action="store_true", help="only the 2,048-token prefill (for profiles)")
     ap.add_argument("--no-graph", action="store_true", help="do not replay decode steps from a HIP graph")
     ap.add_argument("--no-tune", action="store_true", help="do not let TunableOp choose the library's kernels")
     args = ap.parse_args(argv)
@@ -151,6 +152,10 @@ def main(argv=None) -> int:
         torch.cuda.empty_cache()
         return min(times)
 
+    if args.prefill_only:
+        sec = prefill_rate(2048)
+        print(json.dumps({"prefill": {"value": round(2048 / sec, 1), "tokens": 2048, "ms": round(sec * 1e3, 3)}}))
+        return 0
     value, ms_per_step, ctx_mid = decode_rate(args.batch, args.steps, args.warmup)
     need = step_bytes(t, args.batch, ctx_mid, 2 if args.dtype == "bfloat16" else 4)
     achieved = need / (ms_per_step * 1e-3) / 1e9

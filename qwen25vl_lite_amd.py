@@ -9,9 +9,14 @@ import importlib.util
 import os
 import sys
 
+_name = "qwen25vl_lite_amd"
 _dir = os.path.join(os.path.dirname(os.path.abspath(__file__)), "qwen25vl-lite_amd")
 _spec = importlib.util.spec_from_file_location(
-    __name__, os.path.join(_dir, "__init__.py"), submodule_search_locations=[_dir])
+    _name, os.path.join(_dir, "__init__.py"), submodule_search_locations=[_dir])
 _module = importlib.util.module_from_spec(_spec)
-sys.modules[__name__] = _module
+sys.modules[_name] = _module
 _spec.loader.exec_module(_module)
+
+if __name__ == "__main__":          # ``python -m qwen25vl_lite_amd ...`` is the command line
+    from qwen25vl_lite_amd.cli import main
+    raise SystemExit(main())

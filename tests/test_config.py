@@ -136,3 +136,19 @@ def test_engine_config_validation():
                 dict(dtype="float16"), dict(max_num_batched_tokens=0)):
         with pytest.raises(ValueError):
             EngineConfig(**bad)
+
+
+def test_command_line_is_reachable_as_a_module(tmp_path):
+    """``python -m qwen25vl_lite_amd`` is the command line; make-random writes a model folder."""
+    import json
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cfg = tmp_path / "config.json"
+    cfg.write_text(json.dumps(TINY_A))
+    out = tmp_path / "m"
+    res = subprocess.run([sys.executable, "-m", "qwen25vl_lite_amd", "make-random", "--config", str(cfg),
+                          "--out", str(out), "--seed", "3"], cwd=root, capture_output=True, text=True, timeout=120)
+    assert res.returncode == 0, res.stderr
+    assert (out / "config.json").exists() and (out / "model.safetensors").exists()
