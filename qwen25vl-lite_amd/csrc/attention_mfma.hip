@@ -17,11 +17,16 @@
 // 8g .. 8g+7.  Keys are stored [page][kv head][slot][HD] and values transposed,
 // [page][kv head][HD][slot], so both A operands are plain 16-byte loads from the pages.
 //
-// Two kernels use this walk.  With many tiles (prompt portions) every wave owns a tile.  With
-// few tiles (decode) the waves of a block share one tile and merge through LDS; for very long
-// contexts the keys are further split among blocks, whose partial sums a second kernel merges.
+// Two kernels use this arithmetic.  With many tiles (prompt portions) a block owns several tiles
+// per wave and fetches every key block once, through LDS, for all of them.  With few tiles
+// (decode) the waves of a block share one tile, each loading its own key blocks straight into
+// registers, and merge through LDS; for very long contexts the keys are further split among
+// blocks, whose partial sums a second kernel merges.
 #include "common.h"
 
+#ifndef EXP
+#define EXP 0
+#endif
 #ifndef HD
 #error "compile with -DHD=<head size>"
 #endif
@@ -52,6 +57,34 @@ __device__ __forceinline__ uint32_t pack2(float a, float b) {
   return __builtin_bit_cast(uint32_t, v);
 }
 
+// A column's four lanes are r, r + 16, r + 32, r + 48.  v_permlane16_swap exchanges the odd rows
+// of 16 lanes of its first operand with the even rows of its second, v_permlane32_swap the upper
+// half of the first with the lower half of the second: with both operands equal, the two results
+// hold each pair's two values in both lanes of the pair.
+__device__ __forceinline__ float max_over_groups(float v) {
+  const uint32_t b = __builtin_bit_cast(uint32_t, v);
+  const auto x = __builtin_amdgcn_permlane16_swap(b, b, false, false);
+  v = fmaxf(__builtin_bit_cast(float, (uint32_t)x[0]), __builtin_bit_cast(float, (uint32_t)x[1]));
+  const uint32_t c = __builtin_bit_cast(uint32_t, v);
+  const auto y = __builtin_amdgcn_permlane32_swap(c, c, false, false);
+  return fmaxf(__builtin_bit_cast(float, (uint32_t)y[0]), __builtin_bit_cast(float, (uint32_t)y[1]));
+}
+__device__ __forceinline__ float sum_over_groups(float v) {
+  const uint32_t b = __builtin_bit_cast(uint32_t, v);
+  const auto x = __builtin_amdgcn_permlane16_swap(b, b, false, false);
+  v = __builtin_bit_cast(float, (uint32_t)x[0]) + __builtin_bit_cast(float, (uint32_t)x[1]);
+  const uint32_t c = __builtin_bit_cast(uint32_t, v);
+  const auto y = __builtin_amdgcn_permlane32_swap(c, c, false, false);
+  return __builtin_bit_cast(float, (uint32_t)y[0]) + __builtin_bit_cast(float, (uint32_t)y[1]);
+}
+
+// Softmax state of a column.  m is the reference the exponentials are taken against, in the
+// log2 domain (score * scale * log2 e).  It follows the running maximum lazily: it moves only
+// when a block's maximum exceeds it by more than LAZY_LOG2, so the sums are rarely rescaled and
+// no exponential exceeds 2^LAZY_LOG2; softmax does not depend on the reference.  l is this
+// lane's share of the column's sum (its 8 keys of every block); the four lanes of a column are
+// added up once, after the walk (total_sum).
+#define LAZY_LOG2 8.0f
 struct TileState {
   float m, l;
   f32x4_t acc[NT];
@@ -125,47 +158,37 @@ struct Walk {
       }
       // mask and online softmax; this lane holds keys key0 + 8*lg + j of column r.  A block that
       // lies wholly inside what every column of the wave sees needs no mask.
-      float sv[8];
-      float mloc = -INFINITY;
-      if (interior) {
+      float raw[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          sv[j] = ((j < 4) ? s[0][j] : s[1][j - 4]) * scale_log2;
-          mloc = fmaxf(mloc, sv[j]);
-        }
-      } else {
+      for (int j = 0; j < 8; ++j) raw[j] = (j < 4) ? s[0][j] : s[1][j - 4];
+      if (!interior) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           const int key = key0 + 8 * lg + j;
-          const float raw = (j < 4) ? s[0][j] : s[1][j - 4];
           const bool ok = key >= my_lo[t] && key <= my_p[t] && key >= key_begin && key <= key_end;
-          sv[j] = ok ? raw * scale_log2 : -INFINITY;
-          mloc = fmaxf(mloc, sv[j]);
+          raw[j] = ok ? raw[j] : -INFINITY;
         }
       }
-      mloc = fmaxf(mloc, __shfl_xor(mloc, 16, QVL_WAVE));
-      mloc = fmaxf(mloc, __shfl_xor(mloc, 32, QVL_WAVE));
-      const float m_new = fmaxf(st.m, mloc);
-      float alpha = 1.f, psum = 0.f;
+      float mloc = fmaxf(fmaxf(fmaxf(raw[0], raw[1]), fmaxf(raw[2], raw[3])),
+                         fmaxf(fmaxf(raw[4], raw[5]), fmaxf(raw[6], raw[7])));
+      mloc = max_over_groups(mloc) * scale_log2;   // scale_log2 > 0
+      const bool move = mloc > st.m + LAZY_LOG2;   // always at a column's first visible key (m = -inf)
+      const float m_new = move ? mloc : st.m;
+      const float alpha = move ? __builtin_amdgcn_exp2f(st.m - m_new) : 1.f;
+      // a column that has seen no key yet has m = -inf and only -inf scores: against 0 they give 0
+      const float ref = m_new == -INFINITY ? 0.f : m_new;
+      float psum = 0.f;
       float pv[8];
-      if (m_new == -INFINITY) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) pv[j] = 0.f;
-      } else {
-        alpha = __builtin_amdgcn_exp2f(st.m - m_new);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          pv[j] = __builtin_amdgcn_exp2f(sv[j] - m_new);
-          psum += pv[j];
-        }
+      for (int j = 0; j < 8; ++j) {
+        pv[j] = __builtin_amdgcn_exp2f(fmaf(raw[j], scale_log2, -ref));
+        psum += pv[j];
       }
-      psum += __shfl_xor(psum, 16, QVL_WAVE);
-      psum += __shfl_xor(psum, 32, QVL_WAVE);
       st.l = st.l * alpha + psum;
       st.m = m_new;
-      // the running maximum rarely moves after the first blocks: skip the rescaling when no
-      // column of the wave needs it
-      const bool rescale = __any(alpha != 1.f);
+      // the reference rarely moves after the first blocks: skip the rescaling when no column of
+      // the wave needs it
+      const bool rescale = __any(move);
       u32x4_t packed = {pack2(pv[0], pv[1]), pack2(pv[2], pv[3]), pack2(pv[4], pv[5]), pack2(pv[6], pv[7])};
       const bf16x8_t pb = __builtin_bit_cast(bf16x8_t, packed);
       if (rescale) {
@@ -279,9 +302,6 @@ __device__ __forceinline__ void load_q(const bf16_t* __restrict__ q, int nq, con
   }
 }
 
-// Column tiles per wave in the kernel for many tiles: every key block a wave loads serves two tiles.
-#define TILE_CT 2
-
 __device__ __forceinline__ void init_state(TileState& st) {
   st.m = -INFINITY;
   st.l = 0.f;
@@ -289,55 +309,300 @@ __device__ __forceinline__ void init_state(TileState& st) {
   for (int dt = 0; dt < NT; ++dt) st.acc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 }
 
-// tile_ct counts in units of TILE_CT column tiles here.
-__global__ __launch_bounds__(256) void attn_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc,
-                                                        const bf16_t* __restrict__ vc, const int* __restrict__ bt,
-                                                        int table_width, const int* __restrict__ cu_q,
-                                                        const int* __restrict__ ctx_len,
-                                                        const int* __restrict__ tile_req,
-                                                        const int* __restrict__ tile_ct, int num_tiles,
-                                                        bf16_t* __restrict__ out, int nq, int nkv, int ps, int window,
-                                                        float scale) {
-  const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (item >= num_tiles) return;
-  const int kvh = blockIdx.y, g = nq / nkv;
-  const int r = tile_req[item], ct0 = tile_ct[item] * TILE_CT;
-  const int ncols = (cu_q[r + 1] - cu_q[r]) * g;
-  TileInfo t[TILE_CT];
-  bf16x8_t qb[TILE_CT][KS];
-  TileState st[TILE_CT];
-  int my_lo[TILE_CT], my_p[TILE_CT];
-  int lo = 0x7fffffff, hi = -1;
+// ---- many tiles, keys shared through LDS -------------------------------------------------------
+// A block owns BLK_WAVES * BLK_CT consecutive column tiles of one request and one key/value head;
+// wave w carries tiles (cb * BLK_WAVES + w) * BLK_CT .. + BLK_CT - 1.  The block walks the union
+// of its waves' key ranges.  Every 32-key block is fetched from the pages once per block, by all
+// threads together, and laid out in LDS the way the A operands want it, so the four waves share
+// every byte that leaves L2:
+//   K rows in the permuted order of the top of the file (row 16 b + r holds the key of K block b,
+//   row r), each row padded by 16 bytes: the 16 lanes of a row group read 16 different banks;
+//   V^T rows of 32 keys padded to 40: a stride of 5 x 16 bytes is coprime with the 16 bank groups.
+// Two LDS stages: while block i is computed, block i+1 is on its way from registers into the other
+// stage and the loads of block i+2 are in flight; page numbers are fetched one block further ahead.
+#define BLK_WAVES 4
+#if HD <= 128
+#define BLK_CT 2
+#else
+#define BLK_CT 1
+#endif
+#define KROW (HD + 8)
+#define VROW 40
+#define K_CHUNKS (4 * HD)  // 16-byte chunks of a 32-key K block; the V block has as many
+#define CH_PER_THREAD ((K_CHUNKS + 64 * BLK_WAVES - 1) / (64 * BLK_WAVES))
+#define CH_PER_KEY (HD / 8)
+
+struct StageRegs {
+  u32x4_t k[CH_PER_THREAD], v[CH_PER_THREAD];
+};
+// The pages of the two 16-key halves of a block and the slot in the page where each half begins
+// (a page holds a multiple of 16 keys, so a half never straddles pages).  The same for every
+// thread: the compiler keeps these in scalar registers and fetches the table entries once per wave.
+struct StagePages {
+  int page[2], off[2];
+};
+
+// What a thread fetches of every 32-key block: chunk c = tid + 256 j of K is 8 channels of key
+// c / CH_PER_KEY, chunk c of V^T is keys 8 (c % 4) .. + 7 of channel c / 4.  Everything about a
+// chunk's address that does not change from block to block is worked out once (start); the
+// halves' page index and slot move along with the blocks (next_pages is called for consecutive
+// blocks), so the page size is divided by once.
+struct BlockLoader {
+  const bf16_t* kc;
+  const bf16_t* vc;
+  const int* bt;
+  int table_width, ps, tid;
+  size_t page_stride;            // elements of one page over all heads, K and V alike
+  int idx[2], off[2];            // of the next block's halves
+  int k_fixed[CH_PER_THREAD];    // element offset of the chunk in the page when its half begins at slot 0
+  int v_fixed[CH_PER_THREAD];
+  bool k_half[CH_PER_THREAD], v_half;
+
+  __device__ __forceinline__ void start(int kb, int nkv, int kvh) {
+    page_stride = (size_t)nkv * ps * HD;
 #pragma unroll
-  for (int i = 0; i < TILE_CT; ++i) {
-    const bool exists = (ct0 + i) * 16 < ncols;   // the last pair of a request may have one tile only
-    t[i] = tile_info(cu_q, ctx_len, r, exists ? ct0 + i : ct0, g, kvh, window);
+    for (int h = 0; h < 2; ++h) {
+      const int key = (kb << 5) + 16 * h;
+      idx[h] = key / ps;
+      off[h] = key - idx[h] * ps;
+    }
+#pragma unroll
+    for (int j = 0; j < CH_PER_THREAD; ++j) {
+      const int c = tid + j * 64 * BLK_WAVES;
+      const int kk = c < K_CHUNKS ? c / CH_PER_KEY : 0, part = c % CH_PER_KEY;
+      k_half[j] = kk >= 16;
+      k_fixed[j] = (kvh * ps + (kk & 15)) * HD + part * 8;
+      v_fixed[j] = (kvh * HD + (c >> 2)) * ps + 8 * (tid & 1);
+    }
+    v_half = (tid & 2) != 0;
+  }
+  // Pages of the next block; keys past the table or without a page (nobody sees them) read page 0.
+  __device__ __forceinline__ void next_pages(StagePages& pg) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int p = idx[h] < table_width ? bt[idx[h]] : 0;
+      pg.page[h] = p < 0 ? 0 : p;
+      pg.off[h] = off[h];
+      off[h] += 32;  // a page has at least 16 slots: at most two pages further
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        if (off[h] >= ps) {
+          off[h] -= ps;
+          ++idx[h];
+        }
+    }
+  }
+  __device__ __forceinline__ void loads(const StagePages& pg, StageRegs& rg) const {
+    // where each half begins, for K and for V: the same for all threads (scalar arithmetic)
+    const bf16_t* kh[2];
+    const bf16_t* vh[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      kh[h] = kc + (size_t)pg.page[h] * page_stride + pg.off[h] * HD;
+      vh[h] = vc + (size_t)pg.page[h] * page_stride + pg.off[h];
+    }
+    const bf16_t* vpage = v_half ? vh[1] : vh[0];
+#pragma unroll
+    for (int j = 0; j < CH_PER_THREAD; ++j) {
+      const int c = tid + j * 64 * BLK_WAVES;
+      if (c < K_CHUNKS) {
+        rg.k[j] = *reinterpret_cast<const u32x4_t*>((k_half[j] ? kh[1] : kh[0]) + k_fixed[j]);
+        rg.v[j] = *reinterpret_cast<const u32x4_t*>(vpage + v_fixed[j]);
+      }
+    }
+  }
+  __device__ __forceinline__ void to_lds(const StageRegs& rg, bf16_t* ks, bf16_t* vs) const {
+#pragma unroll
+    for (int j = 0; j < CH_PER_THREAD; ++j) {
+      const int c = tid + j * 64 * BLK_WAVES;
+      if (c < K_CHUNKS) {
+        const int kk = c / CH_PER_KEY, part = c - kk * CH_PER_KEY;
+        const int row = 16 * ((kk >> 2) & 1) + 4 * (kk >> 3) + (kk & 3);
+        *reinterpret_cast<u32x4_t*>(ks + row * KROW + part * 8) = rg.k[j];
+        *reinterpret_cast<u32x4_t*>(vs + (c >> 2) * VROW + 8 * (c & 3)) = rg.v[j];
+      }
+    }
+  }
+};
+
+__device__ __forceinline__ void operands_from_lds(const bf16_t* ks, const bf16_t* vs, BlockRegs& rg) {
+  const int lane = threadIdx.x & 63, lg = lane >> 4, r = lane & 15;
+#pragma unroll
+  for (int b = 0; b < 2; ++b)
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      const int d = s * 32 + 8 * lg;
+      rg.k[b][s] = (d < HD) ? load8(ks + (16 * b + r) * KROW + d) : zero8();
+    }
+#pragma unroll
+  for (int dt = 0; dt < NT; ++dt) rg.v[dt] = load8(vs + (dt * 16 + r) * VROW + 8 * lg);
+}
+
+// One entry of the block list for one key/value head.  blk_cb counts in units of
+// BLK_WAVES * BLK_CT column tiles.
+struct BlockShared {
+  __attribute__((aligned(16))) bf16_t k[2][32 * KROW];
+  __attribute__((aligned(16))) bf16_t v[2][HD * VROW];
+  int wave_range[BLK_WAVES][2];
+  int work;
+};
+
+__device__ __forceinline__ void attend_block(BlockShared& sh, int item, int kvh, const bf16_t* __restrict__ q,
+                                             const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
+                                             const int* __restrict__ bt, int table_width,
+                                             const int* __restrict__ cu_q, const int* __restrict__ ctx_len,
+                                             const int* __restrict__ blk_req, const int* __restrict__ blk_cb,
+                                             bf16_t* __restrict__ out, int nq, int nkv, int ps, int window,
+                                             float scale) {
+  const int g = nq / nkv;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int r = blk_req[item], ct0 = (blk_cb[item] * BLK_WAVES + wave) * BLK_CT;
+  const int ncols = (cu_q[r + 1] - cu_q[r]) * g;
+  TileInfo t[BLK_CT];
+  bf16x8_t qb[BLK_CT][KS];
+  TileState st[BLK_CT];
+  int lo = 0x7fffffff, hi = -1;
+  Walk<BLK_CT> w;
+#pragma unroll
+  for (int i = 0; i < BLK_CT; ++i) {
+    const bool exists = (ct0 + i) * 16 < ncols;   // a request's last block may be short of tiles
+    t[i] = tile_info(cu_q, ctx_len, r, exists ? ct0 + i : 0, g, kvh, window);
     if (!exists) { t[i].valid = false; t[i].my_p = -1; }
     load_q(q, nq, t[i], qb[i]);
     init_state(st[i]);
-    my_lo[i] = t[i].my_lo;
-    my_p[i] = t[i].my_p;
+    w.my_lo[i] = t[i].my_lo;
+    w.my_p[i] = t[i].my_p;
     if (exists) {
       lo = t[i].lo_tile < lo ? t[i].lo_tile : lo;
       hi = t[i].hi_tile > hi ? t[i].hi_tile : hi;
     }
   }
-  attend<TILE_CT>(kc, vc, bt + (size_t)r * table_width, table_width, nkv, kvh, ps, qb, my_lo, my_p, scale * LOG2E, lo,
-                  hi, 0, 1, st);
-  const int lg = (threadIdx.x & 63) >> 4;
+  if (lane == 0) {
+    sh.wave_range[wave][0] = lo;
+    sh.wave_range[wave][1] = hi;
+  }
+  __syncthreads();
+  int blo = 0x7fffffff, bhi = -1;
 #pragma unroll
-  for (int i = 0; i < TILE_CT; ++i) {
+  for (int i = 0; i < BLK_WAVES; ++i) {
+    blo = min(blo, sh.wave_range[i][0]);
+    bhi = max(bhi, sh.wave_range[i][1]);
+  }
+  if (bhi < 0) return;  // uniform over the block
+  w.key_begin = lo; w.key_end = hi;
+  w.scale_log2 = scale * LOG2E; w.lg = lane >> 4; w.r = lane & 15;
+  {  // the range every column of this wave sees
+    int a = lo, b = hi;
+#pragma unroll
+    for (int i = 0; i < BLK_CT; ++i)
+      if (w.my_p[i] >= 0) {
+        a = max(a, w.my_lo[i]);
+        b = min(b, w.my_p[i]);
+      }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      a = max(a, __shfl_xor(a, o, QVL_WAVE));
+      b = min(b, __shfl_xor(b, o, QVL_WAVE));
+    }
+    w.all_lo = a;
+    w.all_hi = b;
+  }
+  BlockLoader ld;
+  ld.kc = kc; ld.vc = vc; ld.bt = bt + (size_t)r * table_width;
+  ld.table_width = table_width; ld.ps = ps; ld.tid = threadIdx.x;
+  const int kb0 = blo >> 5, kb_end = bhi >> 5;  // inclusive
+  StagePages pg, pg_next;
+  StageRegs regs;
+  ld.start(kb0, nkv, kvh);
+  ld.next_pages(pg);
+  const StagePages pg0 = pg;
+  ld.loads(pg, regs);
+  if (kb0 + 1 <= kb_end) ld.next_pages(pg);
+  ld.to_lds(regs, sh.k[0], sh.v[0]);
+  if (kb0 + 1 <= kb_end) ld.loads(pg, regs);
+  if (kb0 + 2 <= kb_end) ld.next_pages(pg);
+  __syncthreads();
+  for (int kb = kb0; kb <= kb_end; ++kb) {
+    const int cur = (kb - kb0) & 1;
+    // block kb+1 has had the last computation to arrive: put it into the stage that block kb-1 left
+    if (kb + 1 <= kb_end) ld.to_lds(regs, sh.k[cur ^ 1], sh.v[cur ^ 1]);
+    if (kb + 3 <= kb_end) ld.next_pages(pg_next);
+#if EXP == 1
+    if (kb + 2 <= kb_end) ld.loads(pg0, regs);
+#else
+    if (kb + 2 <= kb_end) ld.loads(pg, regs);
+#endif
+#if EXP == 2
+    if (kb == kb_end) {
+#else
+    if ((kb << 5) + 31 >= lo && (kb << 5) <= hi) {
+#endif
+      BlockRegs ops;
+      operands_from_lds(sh.k[cur], sh.v[cur], ops);
+      w.compute(kb, qb, ops, st);
+    }
+    pg = pg_next;
+    __syncthreads();
+  }
+  const int lg = lane >> 4;
+#pragma unroll
+  for (int i = 0; i < BLK_CT; ++i) {
+    const float total = sum_over_groups(st[i].l);
     if (!t[i].valid) continue;
-    const float inv = 1.0f / st[i].l;
+    const float inv = 1.0f / total;
     bf16_t* orow = out + ((size_t)t[i].token * nq + t[i].head) * HD;
 #pragma unroll
     for (int dt = 0; dt < NT; ++dt) {
       const int d = dt * 16 + 4 * lg;
-      uint2 w;
-      w.x = pack2(st[i].acc[dt][0] * inv, st[i].acc[dt][1] * inv);
-      w.y = pack2(st[i].acc[dt][2] * inv, st[i].acc[dt][3] * inv);
-      *reinterpret_cast<uint2*>(orow + d) = w;
+      uint2 wv;
+      wv.x = pack2(st[i].acc[dt][0] * inv, st[i].acc[dt][1] * inv);
+      wv.y = pack2(st[i].acc[dt][2] * inv, st[i].acc[dt][3] * inv);
+      *reinterpret_cast<uint2*>(orow + d) = wv;
     }
+  }
+}
+
+// The workgroups take (entry, head) pairs from queues in global memory until these are empty: the
+// host lists the entries longest walk first, so the long walks start at once and the short ones
+// fill in behind them, whatever mix of requests the step has.  Workgroups go to the 8 XCDs in
+// turn; when the key/value heads divide 8 there is a queue per head and a workgroup serves the
+// head of its XCD first (that XCD's L2 then holds one head's keys) and the others when its own
+// queue is empty.  queue[i] is the next entry of queue i, queue[QUEUE_DONE] counts the workgroups
+// that have found every queue empty; the last of them puts all counters back to zero for the
+// next launch (launches that share the counters must not overlap).
+#define QUEUE_DONE 8
+#define QUEUE_INTS 16
+#if HD <= 128
+#define BLK_PER_CU 2
+#else
+#define BLK_PER_CU 1
+#endif
+__global__ __launch_bounds__(64 * BLK_WAVES, BLK_PER_CU) void attn_mfma_block_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
+    const int* __restrict__ bt, int table_width, const int* __restrict__ cu_q, const int* __restrict__ ctx_len,
+    const int* __restrict__ blk_req, const int* __restrict__ blk_cb, int num_blocks, bf16_t* __restrict__ out, int nq,
+    int nkv, int ps, int window, float scale, int* __restrict__ queue) {
+  __shared__ BlockShared sh;
+  const bool per_head = 8 % nkv == 0;
+  const int queues = per_head ? nkv : 1;
+  const int per_queue = per_head ? num_blocks : num_blocks * nkv;
+  const int home = (blockIdx.x & 7) % queues;
+  for (int turn = 0; turn < queues; ++turn) {
+    const int qi = (home + turn) % queues;
+    for (;;) {
+      if (threadIdx.x == 0) sh.work = atomicAdd(&queue[qi], 1);
+      __syncthreads();
+      const int work = sh.work;
+      if (work >= per_queue) break;  // uniform over the block; every workgroup gets here for every queue
+      attend_block(sh, per_head ? work : work / nkv, per_head ? qi : work % nkv, q, kc, vc, bt, table_width, cu_q,
+                   ctx_len, blk_req, blk_cb, out, nq, nkv, ps, window, scale);
+      __syncthreads();               // everybody has read sh.work and is done with the stages
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0 && atomicAdd(&queue[QUEUE_DONE], 1) == (int)gridDim.x - 1) {
+    for (int i = 0; i < queues; ++i) atomicExch(&queue[i], 0);  // nobody takes work any more
+    atomicExch(&queue[QUEUE_DONE], 0);
   }
 }
 
@@ -388,9 +653,10 @@ __global__ __launch_bounds__(64 * COOP_WAVES) void attn_mfma_coop_kernel(
   for (int dt = 0; dt < NT; ++dt)
     *reinterpret_cast<float4*>(mine + dt * 16 + 4 * lg) =
         float4{st.acc[dt][0], st.acc[dt][1], st.acc[dt][2], st.acc[dt][3]};
+  const float total = sum_over_groups(st.l);
   if (lg == 0) {
     mine[HD] = st.m;
-    mine[HD + 1] = st.l;
+    mine[HD + 1] = total;
   }
   __syncthreads();
   // merge: thread -> (column, 4 channels); waves are summed in order 0, 1, ...
@@ -469,19 +735,27 @@ static int check_common(int num_tiles, int nq, int nkv, int ps, int table_width)
 }
 
 extern "C" int qvl_attn_mfma_head_dim() { return HD; }
-// Column tiles per entry of the tile list that qvl_attn_mfma expects (qvl_attn_mfma_coop: 1).
-extern "C" int qvl_attn_mfma_tile_ct() { return TILE_CT; }
+// Column tiles per entry of the block list that qvl_attn_mfma_block expects, and how many of its
+// workgroups a compute unit holds at a time.
+extern "C" int qvl_attn_mfma_block_tiles() { return BLK_WAVES * BLK_CT; }
+extern "C" int qvl_attn_mfma_block_per_cu() { return BLK_PER_CU; }
+extern "C" int qvl_attn_mfma_queue_ints() { return QUEUE_INTS; }
 
-extern "C" int qvl_attn_mfma(const void* q, const void* kc, const void* vc, const void* bt, int table_width,
-                             const void* cu_q, const void* ctx_len, const void* tile_req, const void* tile_ct,
-                             int num_tiles, void* out, int nq, int nkv, int ps, int window, float scale,
-                             hipStream_t stream) {
-  const int c = check_common(num_tiles, nq, nkv, ps, table_width);
+extern "C" int qvl_attn_mfma_block(const void* q, const void* kc, const void* vc, const void* bt, int table_width,
+                                   const void* cu_q, const void* ctx_len, const void* blk_req, const void* blk_cb,
+                                   int num_blocks, void* out, int nq, int nkv, int ps, int window, float scale,
+                                   void* queue, int max_workgroups, hipStream_t stream) {
+  // queue: qvl_attn_mfma_queue_ints() ints, zero before the first launch that uses them
+  const int c = check_common(num_blocks, nq, nkv, ps, table_width);
   if (c >= 0) return c;
-  const dim3 grid((num_tiles + 3) / 4, nkv);
-  hipLaunchKernelGGL(attn_mfma_kernel, grid, dim3(256), 0, stream, (const bf16_t*)q, (const bf16_t*)kc,
-                     (const bf16_t*)vc, (const int*)bt, table_width, (const int*)cu_q, (const int*)ctx_len,
-                     (const int*)tile_req, (const int*)tile_ct, num_tiles, (bf16_t*)out, nq, nkv, ps, window, scale);
+  if (!(scale > 0.f) || !queue || max_workgroups <= 0) return QVL_ERR_SHAPE;
+  const long long total = (long long)num_blocks * nkv;
+  if (total > 0x7fffffffLL) return QVL_ERR_LIMIT;
+  const unsigned grid = (unsigned)(total < max_workgroups ? total : max_workgroups);
+  hipLaunchKernelGGL(attn_mfma_block_kernel, dim3(grid), dim3(64 * BLK_WAVES), 0, stream,
+                     (const bf16_t*)q, (const bf16_t*)kc, (const bf16_t*)vc, (const int*)bt, table_width,
+                     (const int*)cu_q, (const int*)ctx_len, (const int*)blk_req, (const int*)blk_cb, num_blocks,
+                     (bf16_t*)out, nq, nkv, ps, window, scale, (int*)queue);
   return qvl_launch_status();
 }
 
@@ -498,6 +772,7 @@ extern "C" int qvl_attn_mfma_coop(const void* q, const void* kc, const void* vc,
   if (c >= 0) return c;
   if (nsplit <= 0 || nsplit > 65535 || (nsplit > 1 && (keys_per_split <= 0 || keys_per_split % 32 || !scratch)))
     return QVL_ERR_SHAPE;
+  if (!(scale > 0.f)) return QVL_ERR_SHAPE;
   hipLaunchKernelGGL(attn_mfma_coop_kernel, dim3(num_tiles, nkv, nsplit), dim3(64 * COOP_WAVES), 0, stream,
                      (const bf16_t*)q, (const bf16_t*)kc, (const bf16_t*)vc, (const int*)bt, table_width,
                      (const int*)cu_q, (const int*)ctx_len, (const int*)tile_req, (const int*)tile_ct, (bf16_t*)out,

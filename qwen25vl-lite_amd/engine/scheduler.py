@@ -66,9 +66,10 @@ class EngineStats:
     prefix_cache_tokens_saved: int = 0
 
 
-@dataclass
+@dataclass(eq=False)
 class Sequence_:
-    """A request in flight (reference cache.py:584-629)."""
+    """A request in flight (reference cache.py:584-629).  Two requests are the same only if they
+    are the same object (membership tests in the queues compare identities, not fields)."""
 
     seq_id: int
     prompt_token_ids: List[int]
@@ -208,7 +209,8 @@ class LLMEngine:
         # 1. decoding requests (one token left), then 2. prompts already admitted
         for decoding in (True, False):
             for seq in list(self.running):
-                if seq not in self.running or (seq.remaining == 1) != decoding or budget <= 0:
+                # a request earlier in this loop may have preempted this one
+                if seq.status != "running" or (seq.remaining == 1) != decoding or budget <= 0:
                     continue
                 n = self._portion(seq, budget)
                 if n <= 0:

@@ -28,22 +28,34 @@ def supports(head_dim: int, dtype: torch.dtype) -> bool:
     return dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= _MAX_HD
 
 
-TILE_CT = 2   # column tiles a wave carries in the kernel for many tiles (TILE_CT in the source)
 
 
-def tiles_for(cu_q, group: int, tile_ct: int = 1) -> Tuple[np.ndarray, np.ndarray]:
-    """``(tile_req, tile_ct)``: for request r with q tokens, ceil(q * group / (16 * tile_ct)) entries."""
+def block_tiles(head_dim: int) -> int:
+    """Column tiles of one entry of the block list (BLK_WAVES * BLK_CT in the source)."""
+    return int(_fn("attention_mfma", "qvl_attn_mfma_block_tiles", [], {"HD": head_dim})())
+
+
+def tiles_for(cu_q, group: int, tile_ct: int = 1, ctx_len=None) -> Tuple[np.ndarray, np.ndarray]:
+    """``(tile_req, tile_ct)``: for request r with q tokens, ceil(q * group / (16 * tile_ct)) entries.
+    With ``ctx_len`` the entries are listed by the last key they see, latest first: the longest
+    walks start first and the short ones fill the compute units as they become free."""
     q = np.diff(np.asarray(cu_q, dtype=np.int64))
-    counts = (q * group + 16 * tile_ct - 1) // (16 * tile_ct)
+    cols = 16 * tile_ct
+    counts = (q * group + cols - 1) // cols
     req = np.repeat(np.arange(len(q), dtype=np.int32), counts)
     starts = np.cumsum(counts) - counts
     ct = (np.arange(int(counts.sum()), dtype=np.int64) - np.repeat(starts, counts)).astype(np.int32)
+    if ctx_len is not None and len(req):
+        last_token = np.minimum(((ct.astype(np.int64) + 1) * cols - 1) // group, q[req] - 1)
+        last_key = np.asarray(ctx_len, dtype=np.int64)[req] - q[req] + last_token
+        order = np.argsort(-last_key, kind="stable")
+        req, ct = req[order], ct[order]
     return req, ct
 
 
 def plan_splits(num_tiles: int, nkv: int, max_ctx: int) -> Tuple[str, int, int]:
-    """``(kernel, nsplit, keys_per_split)``.  ``"tile"``: every wave owns a tile (many tiles, as in
-    prefill).  ``"coop"``: the waves of a block share a tile (few tiles, as in decode); its keys are
+    """``(kernel, nsplit, keys_per_split)``.  ``"tile"``: many tiles, as in prefill: a block owns
+    several tiles per wave and shares the keys through LDS.  ``"coop"``: the waves of a block share a tile (few tiles, as in decode); its keys are
     split among ``nsplit`` blocks when the context is long and the blocks are few."""
     blocks = num_tiles * nkv
     if blocks >= TARGET_BLOCKS:
@@ -56,11 +68,24 @@ def plan_splits(num_tiles: int, nkv: int, max_ctx: int) -> Tuple[str, int, int]:
     return "coop", (max_ctx + 31 + per - 1) // per, per
 
 
-def _step_tiles(step, group: int, tile_ct: int, device):
+_queues = {}
+
+
+def _work_queue(device: torch.device):
+    """Per device: the counters of the block kernel's work queues (it leaves them at zero) and
+    how many workgroups fill the device."""
+    key = torch.device(device).index or 0
+    if key not in _queues:
+        cus = torch.cuda.get_device_properties(device).multi_processor_count
+        _queues[key] = (torch.zeros(16, dtype=torch.int32, device=device), cus)
+    return _queues[key]
+
+
+def _step_tiles(step, group: int, tile_ct: int, device, by_length: bool = False):
     cache = step.derived
-    key = ("tiles", group, tile_ct)
+    key = ("tiles", group, tile_ct, by_length)
     if key not in cache:
-        req, ct = tiles_for(step.cu_q_host, group, tile_ct)
+        req, ct = tiles_for(step.cu_q_host, group, tile_ct, step.ctx_len_host if by_length else None)
         both = torch.from_numpy(np.concatenate([req, ct])).to(device, non_blocking=True)
         cache[key] = (both[:len(req)], both[len(req):], len(req))
     return cache[key]
@@ -84,13 +109,17 @@ def try_attention(q, k_cache, v_cache, block_table, step, num_q_heads: int, wind
     defines = {"HD": hd}
     kind, nsplit, per = plan_splits(num_tiles, nkv, step.max_ctx_len)
     if kind == "tile":
-        tile_req, tile_ct, num_tiles = _step_tiles(step, nq // nkv, TILE_CT, q.device)
+        tile_req, tile_ct, num_tiles = _step_tiles(step, nq // nkv, block_tiles(hd), q.device, by_length=True)
     common = [_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(step.cu_q),
               _ptr(step.ctx_len), _ptr(tile_req), _ptr(tile_ct), num_tiles, _ptr(out)]
     if kind == "tile":
-        fn = _fn("attention_mfma", "qvl_attn_mfma",
-                 [_c_ptr] * 4 + [_c_int] + [_c_ptr] * 4 + [_c_int, _c_ptr] + [_c_int] * 4 + [_c_float, _c_ptr], defines)
-        _check(fn(*common, nq, nkv, ps, int(window or 0), float(scale), _stream()), "paged_attention (matrix cores)")
+        fn = _fn("attention_mfma", "qvl_attn_mfma_block",
+                 [_c_ptr] * 4 + [_c_int] + [_c_ptr] * 4 + [_c_int, _c_ptr] + [_c_int] * 4
+                 + [_c_float, _c_ptr, _c_int, _c_ptr], defines)
+        queue, cus = _work_queue(q.device)
+        per_cu = int(_fn("attention_mfma", "qvl_attn_mfma_block_per_cu", [], defines)())
+        _check(fn(*common, nq, nkv, ps, int(window or 0), float(scale), _ptr(queue), cus * per_cu, _stream()),
+               "paged_attention (matrix cores)")
     else:
         scratch = None
         if nsplit > 1:

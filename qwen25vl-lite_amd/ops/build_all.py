@@ -23,6 +23,7 @@ LIBRARIES = [
     ("attention_mfma", {"HD": 16}),
     ("attention_mfma", {"HD": 48}),
     ("attention_mfma", {"HD": 80}),
+    ("attention_mfma", {"HD": 256}),
 ]
 
 

@@ -118,23 +118,23 @@ def _paged(k, v, ps, pages, dtype, seed):
 ATTN_SHAPES = [(6, 2, 24, None), (5, 1, 48, 40), (8, 8, 16, 7), (14, 2, 128, None), (4, 2, 80, 130)]
 
 
-def _attention_case(dtype, nq, nkv, hd, window):
+def _attention_case(dtype, nq, nkv, hd, window, lens=(333, 17, 64, 1), qlens=(5, 17, 1, 1)):
     """Prompt portions and single tokens of several requests in one call, pages shuffled, stale
     values in every unused slot.  One query and one far key are scaled so that a single score
     dominates: a kernel that misses that key (a page, a window edge) fails by far."""
     torch.manual_seed(nq * hd)
     ps = 16
-    lens = [333, 17, 64, 1]           # context of each request after this step
-    qlens = [5, 17, 1, 1]             # of which the last qlen are this step's tokens
+    lens, qlens = list(lens), list(qlens)   # context of each request after this step; its last qlen tokens are this step's
+    last = lens[0] - 1
     k = [torch.randn(nkv, t, hd).to(dtype).float() for t in lens]
     v = [torch.randn(nkv, t, hd).to(dtype).float() for t in lens]
     q_all = [torch.randn(nq, t, hd) for t in lens]
-    far = 2 if window is None else max(0, 332 - window + 1)      # the first key the last query still sees
+    far = 2 if window is None else max(0, last - window + 1)      # the first key the last query still sees
     kf = k[0][:, far].repeat_interleave(nq // nkv, 0)
-    q_all[0][:, 332] = kf * (30.0 / (kf.pow(2).sum(-1, keepdim=True) * hd ** -0.5))      # that score is 30
+    q_all[0][:, last] = kf * (30.0 / (kf.pow(2).sum(-1, keepdim=True) * hd ** -0.5))      # that score is 30
     q_all = [x.to(dtype).float() for x in q_all]
     scale = hd ** -0.5
-    kc, vc, table = _paged(k, v, ps, 40, dtype, 1)
+    kc, vc, table = _paged(k, v, ps, sum((t + ps - 1) // ps for t in lens) + 11, dtype, 1)
     qs, req, seqpos, want = [], [], [], []
     for r, (t, ql) in enumerate(zip(lens, qlens)):
         full = plain_attention(q_all[r], k[r], v[r], scale, window)      # [nq, t, hd]
@@ -144,8 +144,8 @@ def _attention_case(dtype, nq, nkv, hd, window):
             seqpos.append(p)
             want.append(full[:, p].reshape(-1))
     want = torch.stack(want)
-    # the dominated row (request 0, position 332) really is the far key's value
-    assert torch.allclose(want[4].view(nq, hd), v[0][:, far].repeat_interleave(nq // nkv, 0), atol=1e-3)
+    # the dominated row (request 0, its last position) really is the far key's value
+    assert torch.allclose(want[qlens[0] - 1].view(nq, hd), v[0][:, far].repeat_interleave(nq // nkv, 0), atol=1e-3)
     return dict(q=torch.stack(qs).to(dtype).cuda(), kc=kc.cuda(), vc=vc.cuda(), table=table.cuda(),
                 req=torch.tensor(req, dtype=torch.int32).cuda(), seqpos=torch.tensor(seqpos, dtype=torch.int32).cuda(),
                 want=want, scale=scale, lens=lens, qlens=qlens)
@@ -165,8 +165,8 @@ def test_paged_attention_generic(dtype, nq, nkv, hd, window):
 @pytest.mark.parametrize("split", ["tile", "coop", "coop_split"])
 @pytest.mark.parametrize("nq, nkv, hd, window", [s for s in ATTN_SHAPES if s[2] % 16 == 0])
 def test_paged_attention_matrix_cores(nq, nkv, hd, window, split, monkeypatch):
-    """The matrix-core kernels on the same case: a wave per tile, the waves of a block sharing a
-    tile, and the keys further split among blocks."""
+    """The matrix-core kernels on the same case: blocks that own several tiles and share the keys
+    through LDS, the waves of a block sharing one tile, and the keys further split among blocks."""
     from qwen25vl_lite_amd.ops import attention_mfma
     from qwen25vl_lite_amd.parts import StepContext
     c = _attention_case(torch.bfloat16, nq, nkv, hd, window)
@@ -183,6 +183,31 @@ def test_paged_attention_matrix_cores(nq, nkv, hd, window, split, monkeypatch):
                        dtype=torch.bfloat16)
     out = attention_mfma.try_attention(c["q"], c["kc"], c["vc"], c["table"], step, nq, window, c["scale"])
     assert out is not None
+    err = (out.float().cpu() - c["want"]).abs().max()
+    assert torch.allclose(out.float().cpu(), c["want"], atol=1.5e-2, rtol=2e-2), err
+
+
+@pytest.mark.parametrize("nq, nkv, hd, window", [(28, 4, 128, None), (6, 2, 48, 100), (4, 4, 256, 257), (5, 1, 16, None)])
+def test_paged_attention_long_portions(nq, nkv, hd, window):
+    """Prompt portions long enough for several blocks of several waves per request, next to a
+    short portion and a decoded token: the kernel that shares keys through LDS walks the union of
+    its waves' ranges, with blocks that some of its waves skip."""
+    from qwen25vl_lite_amd.ops import attention_mfma
+    from qwen25vl_lite_amd.parts import StepContext
+    lens, qlens = (413, 150, 90), (380, 3, 1)
+    c = _attention_case(torch.bfloat16, nq, nkv, hd, window, lens, qlens)
+    cu = [0]
+    for ql in qlens:
+        cu.append(cu[-1] + ql)
+    none = torch.zeros(0, dtype=torch.int32).cuda()
+    step = StepContext(num_tokens=cu[-1], num_reqs=len(lens), token_ids=none, positions=none, token_req=c["req"],
+                       token_seqpos=c["seqpos"], cu_q=torch.tensor(cu, dtype=torch.int32).cuda(),
+                       ctx_len=torch.tensor(lens, dtype=torch.int32).cuda(), req_slots=none, groups=[],
+                       logit_rows=none, cu_q_host=cu, ctx_len_host=list(lens), max_q_len=max(qlens),
+                       max_ctx_len=max(lens), dtype=torch.bfloat16)
+    import unittest.mock as mock
+    with mock.patch.object(attention_mfma, "plan_splits", lambda t, n, m: ("tile", 1, 0)):
+        out = attention_mfma.try_attention(c["q"], c["kc"], c["vc"], c["table"], step, nq, window, c["scale"])
     err = (out.float().cpu() - c["want"]).abs().max()
     assert torch.allclose(out.float().cpu(), c["want"], atol=1.5e-2, rtol=2e-2), err
 
