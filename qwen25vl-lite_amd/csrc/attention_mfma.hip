@@ -24,9 +24,6 @@
 // blocks, whose partial sums a second kernel merges.
 #include "common.h"
 
-#ifndef EXP
-#define EXP 0
-#endif
 #ifndef HD
 #error "compile with -DHD=<head size>"
 #endif
@@ -313,28 +310,45 @@ __device__ __forceinline__ void init_state(TileState& st) {
 // A block owns BLK_WAVES * BLK_CT consecutive column tiles of one request and one key/value head;
 // wave w carries tiles (cb * BLK_WAVES + w) * BLK_CT .. + BLK_CT - 1.  The block walks the union
 // of its waves' key ranges.  Every 32-key block is fetched from the pages once per block, by all
-// threads together, and laid out in LDS the way the A operands want it, so the four waves share
+// waves together, and laid out in LDS the way the A operands want it, so the four waves share
 // every byte that leaves L2:
 //   K rows in the permuted order of the top of the file (row 16 b + r holds the key of K block b,
 //   row r), each row padded by 16 bytes: the 16 lanes of a row group read 16 different banks;
 //   V^T rows of 32 keys padded to 40: a stride of 5 x 16 bytes is coprime with the 16 bank groups.
-// Two LDS stages: while block i is computed, block i+1 is on its way from registers into the other
-// stage and the loads of block i+2 are in flight; page numbers are fetched one block further ahead.
+// The data goes from global memory straight into LDS (global_load_lds_dwordx4: lane l of a wave
+// puts its 16 bytes at M0 + 16 l, so one instruction fills 1 KB of a stage and each lane works out
+// which 16 bytes of the pages belong there; lanes on padding fetch a neighbour's bytes again).
+// No register holds data in flight, so BLK_STAGES - 1 blocks are on their way while one is
+// computed.  The loads are issued from inline assembly and waited for with explicit vmcnt values:
+// every wave issues exactly WAVE_LOADS of them per block.
 #define BLK_WAVES 4
 #if HD <= 128
 #define BLK_CT 2
 #else
 #define BLK_CT 1
 #endif
-#define KROW (HD + 8)
+#define BLK_STAGES 4
+#define CH_PER_KEY (HD / 8)                                       // 16-byte chunks of a key
+#define KROW (HD + 8)                                             // elements of a K row in LDS
 #define VROW 40
-#define K_CHUNKS (4 * HD)  // 16-byte chunks of a 32-key K block; the V block has as many
-#define CH_PER_THREAD ((K_CHUNKS + 64 * BLK_WAVES - 1) / (64 * BLK_WAVES))
-#define CH_PER_KEY (HD / 8)
+#define K_LOADS ((32 * (CH_PER_KEY + 1) + 63) / 64)               // 1 KB wave loads that cover the K rows
+#define V_LOADS ((HD * 5 + 63) / 64)
+#define STAGE_LOADS (K_LOADS + V_LOADS)
+#define WAVE_LOADS ((STAGE_LOADS + BLK_WAVES - 1) / BLK_WAVES)
+#define STAGE_ELEMS (STAGE_LOADS * 512)
+#if 2 * WAVE_LOADS > 63
+#error "the in-flight loads of a wave do not fit the vmcnt counter"
+#endif
 
-struct StageRegs {
-  u32x4_t k[CH_PER_THREAD], v[CH_PER_THREAD];
-};
+__device__ __forceinline__ void load16_to_lds(const bf16_t* g, uint32_t lds_byte_address) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds_byte_address) : "memory");
+}
+// Wait until at most n of this wave's loads are outstanding (they finish in order).
+template <int N>
+__device__ __forceinline__ void wait_loads() {
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0f70);
+}
+
 // The pages of the two 16-key halves of a block and the slot in the page where each half begins
 // (a page holds a multiple of 16 keys, so a half never straddles pages).  The same for every
 // thread: the compiler keeps these in scalar registers and fetches the table entries once per wave.
@@ -342,24 +356,29 @@ struct StagePages {
   int page[2], off[2];
 };
 
-// What a thread fetches of every 32-key block: chunk c = tid + 256 j of K is 8 channels of key
-// c / CH_PER_KEY, chunk c of V^T is keys 8 (c % 4) .. + 7 of channel c / 4.  Everything about a
-// chunk's address that does not change from block to block is worked out once (start); the
-// halves' page index and slot move along with the blocks (next_pages is called for consecutive
-// blocks), so the page size is divided by once.
+// Wave w issues the loads t = (w + BLK_WAVES i) mod STAGE_LOADS, i < WAVE_LOADS, of a block (a
+// load may be issued twice: same bytes to the same place).  Load t < K_LOADS fills K slots
+// 64 t .. 64 t + 63, the others V slots; slot q of K is chunk q mod (CH_PER_KEY + 1) of row
+// q / (CH_PER_KEY + 1), slot q of V^T is keys 8 (q mod 5) .. + 7 of channel q / 5.  Everything
+// about a lane's address that does not change from block to block is worked out once (start);
+// the halves' page index and slot move along with the blocks (next_pages is called for
+// consecutive blocks), so the page size is divided by once.
 struct BlockLoader {
   const bf16_t* kc;
   const bf16_t* vc;
   const int* bt;
-  int table_width, ps, tid;
+  int table_width, ps, wave;
   size_t page_stride;            // elements of one page over all heads, K and V alike
   int idx[2], off[2];            // of the next block's halves
-  int k_fixed[CH_PER_THREAD];    // element offset of the chunk in the page when its half begins at slot 0
-  int v_fixed[CH_PER_THREAD];
-  bool k_half[CH_PER_THREAD], v_half;
+  int fixed[WAVE_LOADS];         // element offset of the lane's bytes in the page when its half begins at slot 0
+  uint32_t halves;               // bit i: load i takes the second half's page
+
+  __device__ __forceinline__ int load_index(int i) const { return (wave + BLK_WAVES * i) % STAGE_LOADS; }
 
   __device__ __forceinline__ void start(int kb, int nkv, int kvh) {
+    const int lane = threadIdx.x & 63;
     page_stride = (size_t)nkv * ps * HD;
+    halves = 0;
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const int key = (kb << 5) + 16 * h;
@@ -367,14 +386,26 @@ struct BlockLoader {
       off[h] = key - idx[h] * ps;
     }
 #pragma unroll
-    for (int j = 0; j < CH_PER_THREAD; ++j) {
-      const int c = tid + j * 64 * BLK_WAVES;
-      const int kk = c < K_CHUNKS ? c / CH_PER_KEY : 0, part = c % CH_PER_KEY;
-      k_half[j] = kk >= 16;
-      k_fixed[j] = (kvh * ps + (kk & 15)) * HD + part * 8;
-      v_fixed[j] = (kvh * HD + (c >> 2)) * ps + 8 * (tid & 1);
+    for (int i = 0; i < WAVE_LOADS; ++i) {
+      const int t = load_index(i);
+      if (t < K_LOADS) {
+        const int slot = 64 * t + lane;
+        int row = slot / (CH_PER_KEY + 1), part = slot - row * (CH_PER_KEY + 1);
+        row = row < 32 ? row : 31;
+        part = part < CH_PER_KEY ? part : CH_PER_KEY - 1;
+        const int b = row >> 4, r = row & 15;
+        const int kk = 8 * (r >> 2) + 4 * b + (r & 3);   // the key of LDS row 16 b + r
+        halves |= (kk >= 16 ? 1u : 0u) << i;
+        fixed[i] = (kvh * ps + (kk & 15)) * HD + part * 8;
+      } else {
+        const int slot = 64 * (t - K_LOADS) + lane;
+        int row = slot / 5, part = slot - row * 5;
+        row = row < HD ? row : HD - 1;
+        part = part < 4 ? part : 3;
+        halves |= (part >= 2 ? 1u : 0u) << i;
+        fixed[i] = (kvh * HD + row) * ps + 8 * (part & 1);
+      }
     }
-    v_half = (tid & 2) != 0;
   }
   // Pages of the next block; keys past the table or without a page (nobody sees them) read page 0.
   __device__ __forceinline__ void next_pages(StagePages& pg) {
@@ -392,7 +423,8 @@ struct BlockLoader {
         }
     }
   }
-  __device__ __forceinline__ void loads(const StagePages& pg, StageRegs& rg) const {
+  // Issue this wave's loads of the block with pages pg into the stage at LDS byte address stage.
+  __device__ __forceinline__ void issue(const StagePages& pg, uint32_t stage) const {
     // where each half begins, for K and for V: the same for all threads (scalar arithmetic)
     const bf16_t* kh[2];
     const bf16_t* vh[2];
@@ -401,26 +433,12 @@ struct BlockLoader {
       kh[h] = kc + (size_t)pg.page[h] * page_stride + pg.off[h] * HD;
       vh[h] = vc + (size_t)pg.page[h] * page_stride + pg.off[h];
     }
-    const bf16_t* vpage = v_half ? vh[1] : vh[0];
 #pragma unroll
-    for (int j = 0; j < CH_PER_THREAD; ++j) {
-      const int c = tid + j * 64 * BLK_WAVES;
-      if (c < K_CHUNKS) {
-        rg.k[j] = *reinterpret_cast<const u32x4_t*>((k_half[j] ? kh[1] : kh[0]) + k_fixed[j]);
-        rg.v[j] = *reinterpret_cast<const u32x4_t*>(vpage + v_fixed[j]);
-      }
-    }
-  }
-  __device__ __forceinline__ void to_lds(const StageRegs& rg, bf16_t* ks, bf16_t* vs) const {
-#pragma unroll
-    for (int j = 0; j < CH_PER_THREAD; ++j) {
-      const int c = tid + j * 64 * BLK_WAVES;
-      if (c < K_CHUNKS) {
-        const int kk = c / CH_PER_KEY, part = c - kk * CH_PER_KEY;
-        const int row = 16 * ((kk >> 2) & 1) + 4 * (kk >> 3) + (kk & 3);
-        *reinterpret_cast<u32x4_t*>(ks + row * KROW + part * 8) = rg.k[j];
-        *reinterpret_cast<u32x4_t*>(vs + (c >> 2) * VROW + 8 * (c & 3)) = rg.v[j];
-      }
+    for (int i = 0; i < WAVE_LOADS; ++i) {
+      const int t = load_index(i);
+      const bool second = (halves >> i) & 1u;
+      const bf16_t* base = t < K_LOADS ? (second ? kh[1] : kh[0]) : (second ? vh[1] : vh[0]);
+      load16_to_lds(base + fixed[i], __builtin_amdgcn_readfirstlane(stage + 1024u * t));
     }
   }
 };
@@ -441,8 +459,7 @@ __device__ __forceinline__ void operands_from_lds(const bf16_t* ks, const bf16_t
 // One entry of the block list for one key/value head.  blk_cb counts in units of
 // BLK_WAVES * BLK_CT column tiles.
 struct BlockShared {
-  __attribute__((aligned(16))) bf16_t k[2][32 * KROW];
-  __attribute__((aligned(16))) bf16_t v[2][HD * VROW];
+  __attribute__((aligned(16))) bf16_t stage[BLK_STAGES][STAGE_ELEMS];   // K rows, then V^T rows
   int wave_range[BLK_WAVES][2];
   int work;
 };
@@ -455,7 +472,7 @@ __device__ __forceinline__ void attend_block(BlockShared& sh, int item, int kvh,
                                              bf16_t* __restrict__ out, int nq, int nkv, int ps, int window,
                                              float scale) {
   const int g = nq / nkv;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int r = blk_req[item], ct0 = (blk_cb[item] * BLK_WAVES + wave) * BLK_CT;
   const int ncols = (cu_q[r + 1] - cu_q[r]) * g;
   TileInfo t[BLK_CT];
@@ -489,6 +506,8 @@ __device__ __forceinline__ void attend_block(BlockShared& sh, int item, int kvh,
     bhi = max(bhi, sh.wave_range[i][1]);
   }
   if (bhi < 0) return;  // uniform over the block
+  blo = __builtin_amdgcn_readfirstlane(blo);
+  bhi = __builtin_amdgcn_readfirstlane(bhi);
   w.key_begin = lo; w.key_end = hi;
   w.scale_log2 = scale * LOG2E; w.lg = lane >> 4; w.r = lane & 15;
   {  // the range every column of this wave sees
@@ -509,40 +528,42 @@ __device__ __forceinline__ void attend_block(BlockShared& sh, int item, int kvh,
   }
   BlockLoader ld;
   ld.kc = kc; ld.vc = vc; ld.bt = bt + (size_t)r * table_width;
-  ld.table_width = table_width; ld.ps = ps; ld.tid = threadIdx.x;
-  const int kb0 = blo >> 5, kb_end = bhi >> 5;  // inclusive
-  StagePages pg, pg_next;
-  StageRegs regs;
+  ld.table_width = table_width; ld.ps = ps; ld.wave = wave;
+  const int kb0 = blo >> 5, nblk = (bhi >> 5) - kb0 + 1;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)&sh.stage[0][0];
+  StagePages pg;
   ld.start(kb0, nkv, kvh);
   ld.next_pages(pg);
-  const StagePages pg0 = pg;
-  ld.loads(pg, regs);
-  if (kb0 + 1 <= kb_end) ld.next_pages(pg);
-  ld.to_lds(regs, sh.k[0], sh.v[0]);
-  if (kb0 + 1 <= kb_end) ld.loads(pg, regs);
-  if (kb0 + 2 <= kb_end) ld.next_pages(pg);
-  __syncthreads();
-  for (int kb = kb0; kb <= kb_end; ++kb) {
-    const int cur = (kb - kb0) & 1;
-    // block kb+1 has had the last computation to arrive: put it into the stage that block kb-1 left
-    if (kb + 1 <= kb_end) ld.to_lds(regs, sh.k[cur ^ 1], sh.v[cur ^ 1]);
-    if (kb + 3 <= kb_end) ld.next_pages(pg_next);
-#if EXP == 1
-    if (kb + 2 <= kb_end) ld.loads(pg0, regs);
-#else
-    if (kb + 2 <= kb_end) ld.loads(pg, regs);
-#endif
-#if EXP == 2
-    if (kb == kb_end) {
-#else
+  // the queries are in their registers before the first asynchronous load is issued: from here to
+  // the end of the walk the compiler finds nothing of its own to wait for in vmcnt
+  wait_loads<0>();
+  int issued = 0;   // blocks whose loads are issued; pg holds the pages of the next one
+#pragma unroll
+  for (int d = 0; d < BLK_STAGES - 1; ++d)
+    if (issued < nblk) {
+      ld.issue(pg, lds0 + (uint32_t)(issued % BLK_STAGES) * (STAGE_ELEMS * 2));
+      ++issued;
+      if (issued < nblk) ld.next_pages(pg);
+    }
+  for (int i = 0; i < nblk; ++i) {
+    // block i has landed when only the loads of the blocks issued after it are outstanding
+    const int later = issued - 1 - i;
+    if (later >= 2) wait_loads<2 * WAVE_LOADS>();
+    else if (later == 1) wait_loads<WAVE_LOADS>();
+    else wait_loads<0>();
+    __syncthreads();   // everybody's part of block i is there, and everybody has left block i - 1
+    if (issued < nblk) {
+      ld.issue(pg, lds0 + (uint32_t)(issued % BLK_STAGES) * (STAGE_ELEMS * 2));   // into the stage of block i - 1
+      ++issued;
+      if (issued < nblk) ld.next_pages(pg);
+    }
+    const int kb = kb0 + i;
     if ((kb << 5) + 31 >= lo && (kb << 5) <= hi) {
-#endif
+      const bf16_t* stage = sh.stage[i % BLK_STAGES];
       BlockRegs ops;
-      operands_from_lds(sh.k[cur], sh.v[cur], ops);
+      operands_from_lds(stage, stage + K_LOADS * 512, ops);
       w.compute(kb, qb, ops, st);
     }
-    pg = pg_next;
-    __syncthreads();
   }
   const int lg = lane >> 4;
 #pragma unroll
@@ -592,7 +613,7 @@ __global__ __launch_bounds__(64 * BLK_WAVES, BLK_PER_CU) void attn_mfma_block_ke
     for (;;) {
       if (threadIdx.x == 0) sh.work = atomicAdd(&queue[qi], 1);
       __syncthreads();
-      const int work = sh.work;
+      const int work = __builtin_amdgcn_readfirstlane(sh.work);   // the same for all: keep it scalar
       if (work >= per_queue) break;  // uniform over the block; every workgroup gets here for every queue
       attend_block(sh, per_head ? work : work / nkv, per_head ? qi : work % nkv, q, kc, vc, bt, table_width, cu_q,
                    ctx_len, blk_req, blk_cb, out, nq, nkv, ps, window, scale);
