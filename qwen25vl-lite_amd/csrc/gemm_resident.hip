@@ -4,7 +4,10 @@
 // between two products a short kernel of its own costs more than its arithmetic (its code and
 // data have just been flushed from the caches by the weights).
 //
-// A block of 16 waves owns row tiles of W (16 rows = 16 outputs each; tile, tile + gridDim.x, ...).
+// A block of 16 waves owns row tiles of W (tile, tile + gridDim.x, ...).  A tile has `rows` <= 16
+// rows of W (= outputs); the host picks `rows` so that the tiles divide evenly among the compute
+// units (3584 outputs on 256 units: 256 tiles of 14 rather than 224 of 16), the matrix-core tile's
+// other rows stay zero.
 // Wave w covers the 256 values of K from 256 w on, as the A operand (W rows) and B operand (X
 // rows) of v_mfma_f32_16x16x32_bf16; the 16 waves' sums meet in LDS and are added in wave order.
 // If K fits one pass (K <= 4096) the X operand stays in registers for all of the block's tiles and
@@ -44,6 +47,7 @@ struct ResidentArgs {
   void* out;
   int ldo;
   int M, N, K, ntiles;
+  int rows;              // rows of W per tile, 1..16 (16 with EPI_SWIGLU)
 };
 
 __device__ __forceinline__ bf16x8_t load8(const bf16_t* p) {
@@ -119,8 +123,8 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
     }
   };
   auto load_w = [&](int tile, int k0, bf16x8_t* a) {
-    const bool row_ok = tile * 16 + r < p.N;
-    const bf16_t* wrow = p.W + (size_t)(row_ok ? tile * 16 + r : 0) * p.ldw;
+    const bool row_ok = r < p.rows && tile * p.rows + r < p.N;
+    const bf16_t* wrow = p.W + (size_t)(row_ok ? tile * p.rows + r : 0) * p.ldw;
 #pragma unroll
     for (int u = 0; u < RK; ++u) {
       const int k = k0 + k_lane + u * 32;
@@ -134,7 +138,7 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
     __syncthreads();
     if (threadIdx.x < 256) {
       const int e = threadIdx.x;
-      const int m = e >> 4, nl = e & 15, n = tile * 16 + nl;
+      const int m = e >> 4, nl = e & 15, n = tile * p.rows + nl;
       float sum = 0.f;
 #pragma unroll
       for (int w = 0; w < RW; ++w) sum += red[w][nl * 16 + m];
@@ -144,7 +148,7 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
           bf16_t* o = reinterpret_cast<bf16_t*>(p.out);
           o[(size_t)m * p.ldo + tile * 8 + nl] = f32_to_bf16((sum / (1.0f + expf(-sum))) * up);
         }
-      } else if (m < p.M && n < p.N) {
+      } else if (m < p.M && nl < p.rows && n < p.N) {
         if (p.bias) sum += p.bias[n];
         if (EPI == EPI_RESIDUAL) {
           float* o = reinterpret_cast<float*>(p.out);
@@ -226,7 +230,15 @@ extern "C" int qvl_gemm_resident(const void* x, int ldx, const void* h, int ldh,
   ResidentArgs p;
   p.X = (const bf16_t*)x; p.ldx = ldx; p.H = (const float*)h; p.ldh = ldh; p.norm_w = (const float*)norm_w;
   p.eps = eps; p.W = (const bf16_t*)W; p.ldw = ldw; p.bias = (const float*)bias; p.out = out; p.ldo = ldo;
-  p.M = M; p.N = N; p.K = K; p.ntiles = (N + 15) / 16;
+  p.M = M; p.N = N; p.K = K;
+  // as many rounds of tiles as 16-row tiles need, with rows per tile cut down to what fills them evenly
+  p.rows = 16;
+  if (epilogue != EPI_SWIGLU) {
+    const long long per_round = 16LL * max_blocks;
+    const long long rounds = (N + per_round - 1) / per_round;
+    p.rows = (int)((N + rounds * max_blocks - 1) / (rounds * max_blocks));
+  }
+  p.ntiles = (N + p.rows - 1) / p.rows;
 #define QVL_RES(TO, EPI)                                                    \
   do {                                                                      \
     if (norm) launch<TO, PRO_NORM, EPI>(p, max_blocks, stream);             \
