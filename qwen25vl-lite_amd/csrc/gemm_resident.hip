@@ -66,13 +66,16 @@ template <typename TO, int PRO, int EPI, bool ONE_PASS>
 __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) {
   __shared__ float red[RW][256];
   __shared__ float rowsq[RW][16];
+  __shared__ __attribute__((aligned(16))) float gains[PRO == PRO_NORM ? RW : 1][RK * 32];   // norm weights of each wave's columns
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lg = lane >> 4, r = lane & 15;
   const int k_lane = wave * RK * 32 + 8 * lg;  // first K index of this lane within a pass
   const bool m_ok = r < p.M;
 
   // ---- the X operand of one pass ------------------------------------------------------------
-  auto load_x = [&](int k0, bf16x8_t* xb) {
+  // first_w issues the block's first W loads at the point of the prologue where they fit best
+  auto load_x = [&](int k0, bf16x8_t* xb, auto first_w) {
     if (PRO == PRO_PLAIN) {
+      first_w();   // W first: it is the long wait
       const bf16_t* xrow = p.X + (size_t)(m_ok ? r : 0) * p.ldx;
 #pragma unroll
       for (int u = 0; u < RK; ++u) {
@@ -81,10 +84,12 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
       }
     } else {
       // rmsnorm of the float32 rows: this pass covers all of K (ONE_PASS), so the block's waves
-      // hold whole rows between them
+      // hold whole rows between them.  Loads return in the order they are issued: the rows and
+      // the norm weights are asked for first and W (by first_w) right behind them, so the
+      // statistics and the scaling run while W is still on its way.  A lane fetches 4 of its
+      // wave's 256 norm weights; they reach the lanes that need them through LDS.
       const float* hrow = p.H + (size_t)(m_ok ? r : 0) * p.ldh;
       float4 v[RK][2];
-      float ss = 0.f;
 #pragma unroll
       for (int u = 0; u < RK; ++u) {
         const int k = k_lane + u * 32;
@@ -94,12 +99,19 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
         } else {
           v[u][0] = v[u][1] = float4{0.f, 0.f, 0.f, 0.f};
         }
+      }
+      const int kg = wave * RK * 32 + 4 * lane;
+      const float4 g4 = kg < p.K ? *reinterpret_cast<const float4*>(p.norm_w + kg) : float4{0.f, 0.f, 0.f, 0.f};
+      first_w();
+      float ss = 0.f;
+#pragma unroll
+      for (int u = 0; u < RK; ++u)
         ss += v[u][0].x * v[u][0].x + v[u][0].y * v[u][0].y + v[u][0].z * v[u][0].z + v[u][0].w * v[u][0].w +
               v[u][1].x * v[u][1].x + v[u][1].y * v[u][1].y + v[u][1].z * v[u][1].z + v[u][1].w * v[u][1].w;
-      }
       ss += __shfl_xor(ss, 16, QVL_WAVE);
       ss += __shfl_xor(ss, 32, QVL_WAVE);
       if (lg == 0) rowsq[wave][r] = ss;
+      *reinterpret_cast<float4*>(&gains[wave][4 * lane]) = g4;
       __syncthreads();
       float total = 0.f;
 #pragma unroll
@@ -109,8 +121,8 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
       for (int u = 0; u < RK; ++u) {
         const int k = k_lane + u * 32;
         if (k < p.K) {
-          const float4 g0 = *reinterpret_cast<const float4*>(p.norm_w + k);
-          const float4 g1 = *reinterpret_cast<const float4*>(p.norm_w + k + 4);
+          const float4 g0 = *reinterpret_cast<const float4*>(&gains[wave][8 * lg + u * 32]);
+          const float4 g1 = *reinterpret_cast<const float4*>(&gains[wave][8 * lg + u * 32 + 4]);
           u32x4_t o = {pack2((v[u][0].x * rs) * g0.x, (v[u][0].y * rs) * g0.y),
                        pack2((v[u][0].z * rs) * g0.z, (v[u][0].w * rs) * g0.w),
                        pack2((v[u][1].x * rs) * g1.x, (v[u][1].y * rs) * g1.y),
@@ -171,8 +183,7 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
     bf16x8_t xb[RK];
     bf16x8_t a[2][RK];
     int tile = blockIdx.x;
-    if (tile < p.ntiles) load_w(tile, 0, a[0]);  // W first: it does not wait for the norm's barrier
-    load_x(0, xb);
+    load_x(0, xb, [&] { if (tile < p.ntiles) load_w(tile, 0, a[0]); });
     for (; tile < p.ntiles; tile += 2 * gridDim.x) {
       const int t1 = tile + gridDim.x, t2 = tile + 2 * gridDim.x;
       if (t1 < p.ntiles) load_w(t1, 0, a[1]);
@@ -186,8 +197,7 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
       f32x4_t acc = zero;
       for (int k0 = 0; k0 < p.K; k0 += PASS_K) {
         bf16x8_t xb[RK], a[RK];
-        load_w(tile, k0, a);
-        load_x(k0, xb);
+        load_x(k0, xb, [&] { load_w(tile, k0, a); });
         acc = product(a, xb, acc);
       }
       finish(tile, acc);
