@@ -229,6 +229,30 @@ extern "C" int qvl_rope_kv_write(const void* x, int x_stride, const void* bias, 
 }
 
 // ---------------------------------------------------------------------------------------
+// The rotation's cosines and sines of a step, for kernels that rotate without computing angles:
+// out[n, f] = (cos, sin) of pos[freq_row[f], n] * inv_freq[f], or (1, 0) where freq_row[f] < 0.
+// ---------------------------------------------------------------------------------------
+__global__ void rope_table_kernel(const int* __restrict__ pos, int pos_stride, const float* __restrict__ inv_freq,
+                                  const int* __restrict__ freq_row, float2* __restrict__ out, int rot_half) {
+  const int n = blockIdx.x;
+  for (int f = threadIdx.x; f < rot_half; f += blockDim.x) {
+    const int row = freq_row[f];
+    float c = 1.f, s = 0.f;
+    if (row >= 0) sincosf((float)pos[(size_t)row * pos_stride + n] * inv_freq[f], &s, &c);
+    out[(size_t)n * rot_half + f] = float2{c, s};
+  }
+}
+
+extern "C" int qvl_rope_table(const void* pos, int pos_stride, const void* inv_freq, const void* freq_row, void* out,
+                              int N, int rot_half, hipStream_t stream) {
+  if (N <= 0 || rot_half <= 0) return QVL_OK;
+  if (pos_stride < N) return QVL_ERR_SHAPE;
+  hipLaunchKernelGGL(rope_table_kernel, dim3(N), dim3(64), 0, stream, (const int*)pos, pos_stride,
+                     (const float*)inv_freq, (const int*)freq_row, (float2*)out, rot_half);
+  return qvl_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------
 // SwiGLU: out[n, i] = silu(gate[n, i]) * up[n, i],  silu(z) = z / (1 + exp(-z))  (reference text.py:66)
 // x[n] holds gate and up: plain, gate in columns 0..I-1 and up in I..2I-1; grouped, alternating
 // groups of 8 gate columns and 8 up columns (feature i: gate at 16 (i/8) + i%8, up 8 further),

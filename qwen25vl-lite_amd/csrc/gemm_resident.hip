@@ -20,6 +20,10 @@
 //   epilogue  EPI_RESIDUAL  out += product, out being the float32 residual
 //             EPI_SWIGLU    W's rows come in groups of 8 gate rows, 8 up rows; out[M, N/2] =
 //                           silu(gate) * up, in bfloat16
+//             EPI_ROPE      W is the stacked query | key | value projection.  A tile of a query or
+//                           key head takes 8 channels and the 8 channels they are rotated with
+//                           (half a head further), so the rotation happens here; queries are
+//                           written out, keys and values go straight into their page slots
 #include "common.h"
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
@@ -32,7 +36,7 @@ typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 #define PASS_K (RW * RK * 32)
 
 enum { PRO_PLAIN = 0, PRO_NORM = 1 };
-enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2 };
+enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2, EPI_ROPE = 3 };
 
 struct ResidentArgs {
   const bf16_t* X;       // PRO_PLAIN: [M, K]
@@ -47,7 +51,16 @@ struct ResidentArgs {
   void* out;
   int ldo;
   int M, N, K, ntiles;
-  int rows;              // rows of W per tile, 1..16 (16 with EPI_SWIGLU)
+  int rows;              // rows of W per tile, 1..16 (16 with EPI_SWIGLU and EPI_ROPE)
+  // EPI_ROPE: W rows are nq query heads, nkv key heads, nkv value heads of hd channels each
+  // (hd a multiple of 16, rotation over the whole head in pairs (f, f + hd/2))
+  const float* cs;       // [M, hd/2, 2] cosine and sine of each token's angle at each frequency
+  const int* slot;       // [M] flat slot of each token in the cache (page * ps + offset), -1: none
+  bf16_t* q_out;         // [M, nq hd]
+  bf16_t* kc;            // [pages, nkv, ps, hd]
+  bf16_t* vc;            // [pages, nkv, hd, ps]
+  int nq, nkv, hd, ps;
+  int pair_tiles;        // tiles of query and key heads (16 rows each); value tiles of `rows` rows follow
 };
 
 __device__ __forceinline__ bf16x8_t load8(const bf16_t* p) {
@@ -134,23 +147,62 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
       }
     }
   };
+  // the rows of a tile, and the row of W behind row i of a tile
+  auto tile_rows = [&](int tile) { return (EPI == EPI_ROPE && tile < p.pair_tiles) ? 16 : p.rows; };
+  auto w_row = [&](int tile, int i) {
+    if (EPI == EPI_ROPE) {
+      if (tile < p.pair_tiles) {  // 8 channels of a query or key head and the 8 they are rotated with
+        const int tph = p.hd >> 4, head = tile / tph, sub = tile - head * tph;
+        return head * p.hd + 8 * sub + (i & 7) + (i >> 3) * (p.hd >> 1);
+      }
+      return (p.nq + p.nkv) * p.hd + (tile - p.pair_tiles) * p.rows + i;   // value rows
+    }
+    return tile * p.rows + i;
+  };
   auto load_w = [&](int tile, int k0, bf16x8_t* a) {
-    const bool row_ok = r < p.rows && tile * p.rows + r < p.N;
-    const bf16_t* wrow = p.W + (size_t)(row_ok ? tile * p.rows + r : 0) * p.ldw;
+    const int row = w_row(tile, r);
+    const bool row_ok = r < tile_rows(tile) && row < p.N;
+    const bf16_t* wrow = p.W + (size_t)(row_ok ? row : 0) * p.ldw;
 #pragma unroll
     for (int u = 0; u < RK; ++u) {
       const int k = k0 + k_lane + u * 32;
       a[u] = (row_ok && k < p.K) ? load8(wrow + k) : zero8();
     }
   };
+  // What the epilogue of a tile reads from memory, for the element (m, nl) this thread finishes.
+  // Loads return in the order they are issued, so these are asked for before the W loads of the
+  // next tile: waiting for them must not wait for those.
+  struct Epi {
+    float bias, old;
+    float2 cs;
+    int slot;
+  };
+  auto epi_load = [&](int tile) {
+    Epi e;
+    e.bias = e.old = 0.f;
+    e.cs = float2{1.f, 0.f};
+    e.slot = -1;
+    if (threadIdx.x >= 256 || EPI == EPI_SWIGLU) return e;
+    const int m = threadIdx.x >> 4, nl = threadIdx.x & 15, n = w_row(tile, nl);
+    if (m >= p.M || nl >= tile_rows(tile) || n >= p.N) return e;
+    if (p.bias) e.bias = p.bias[n];
+    if (EPI == EPI_RESIDUAL) e.old = reinterpret_cast<const float*>(p.out)[(size_t)m * p.ldo + n];
+    if (EPI == EPI_ROPE) {
+      const int head = n / p.hd, d = n - head * p.hd, half = p.hd >> 1;
+      if (head < p.nq + p.nkv)
+        e.cs = *reinterpret_cast<const float2*>(p.cs + ((size_t)m * half + (d < half ? d : d - half)) * 2);
+      if (head >= p.nq) e.slot = p.slot[m];
+    }
+    return e;
+  };
   // ---- merge the waves' sums of one tile and write the result -----------------------------------
-  auto finish = [&](int tile, const f32x4_t& acc) {
+  auto finish = [&](int tile, const f32x4_t& acc, const Epi& epi) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) red[wave][(4 * lg + i) * 16 + r] = acc[i];
     __syncthreads();
     if (threadIdx.x < 256) {
       const int e = threadIdx.x;
-      const int m = e >> 4, nl = e & 15, n = tile * p.rows + nl;
+      const int m = e >> 4, nl = e & 15, n = w_row(tile, nl);
       float sum = 0.f;
 #pragma unroll
       for (int w = 0; w < RW; ++w) sum += red[w][nl * 16 + m];
@@ -160,11 +212,29 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
           bf16_t* o = reinterpret_cast<bf16_t*>(p.out);
           o[(size_t)m * p.ldo + tile * 8 + nl] = f32_to_bf16((sum / (1.0f + expf(-sum))) * up);
         }
+      } else if (EPI == EPI_ROPE) {
+        sum += epi.bias;
+        const float other = __shfl_xor(sum, 8, QVL_WAVE);   // the channel this one is rotated with
+        const int head = n / p.hd, d = n - head * p.hd;
+        if (m < p.M && nl < tile_rows(tile) && n < p.N) {
+          // (cos, sin) is (1, 0) for value heads; rows 0..7 of a rotated tile are the first halves
+          const float val = (nl < 8 || head >= p.nq + p.nkv) ? sum * epi.cs.x - other * epi.cs.y
+                                                              : sum * epi.cs.x + other * epi.cs.y;
+          if (head < p.nq) {
+            p.q_out[((size_t)m * p.nq + head) * p.hd + d] = f32_to_bf16(val);
+          } else if (epi.slot >= 0) {
+            const size_t page = (size_t)(epi.slot / p.ps), off = (size_t)(epi.slot % p.ps);
+            if (head < p.nq + p.nkv)
+              p.kc[((page * p.nkv + (head - p.nq)) * p.ps + off) * p.hd + d] = f32_to_bf16(val);
+            else
+              p.vc[((page * p.nkv + (head - p.nq - p.nkv)) * p.hd + d) * p.ps + off] = f32_to_bf16(val);
+          }
+        }
       } else if (m < p.M && nl < p.rows && n < p.N) {
-        if (p.bias) sum += p.bias[n];
+        sum += epi.bias;
         if (EPI == EPI_RESIDUAL) {
           float* o = reinterpret_cast<float*>(p.out);
-          o[(size_t)m * p.ldo + n] += sum;
+          o[(size_t)m * p.ldo + n] = epi.old + sum;
         } else {
           stf<TO>(reinterpret_cast<TO*>(p.out) + (size_t)m * p.ldo + n, sum);
         }
@@ -186,21 +256,24 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
     load_x(0, xb, [&] { if (tile < p.ntiles) load_w(tile, 0, a[0]); });
     for (; tile < p.ntiles; tile += 2 * gridDim.x) {
       const int t1 = tile + gridDim.x, t2 = tile + 2 * gridDim.x;
+      const Epi e0 = epi_load(tile);
       if (t1 < p.ntiles) load_w(t1, 0, a[1]);
-      finish(tile, product(a[0], xb, zero));
+      finish(tile, product(a[0], xb, zero), e0);
       if (t1 >= p.ntiles) break;
+      const Epi e1 = epi_load(t1);
       if (t2 < p.ntiles) load_w(t2, 0, a[0]);
-      finish(t1, product(a[1], xb, zero));
+      finish(t1, product(a[1], xb, zero), e1);
     }
   } else {
     for (int tile = blockIdx.x; tile < p.ntiles; tile += gridDim.x) {
       f32x4_t acc = zero;
+      const Epi e = epi_load(tile);
       for (int k0 = 0; k0 < p.K; k0 += PASS_K) {
         bf16x8_t xb[RK], a[RK];
         load_x(k0, xb, [&] { load_w(tile, k0, a); });
         acc = product(a, xb, acc);
       }
-      finish(tile, acc);
+      finish(tile, acc, e);
     }
   }
 }
@@ -241,6 +314,8 @@ extern "C" int qvl_gemm_resident(const void* x, int ldx, const void* h, int ldh,
   p.X = (const bf16_t*)x; p.ldx = ldx; p.H = (const float*)h; p.ldh = ldh; p.norm_w = (const float*)norm_w;
   p.eps = eps; p.W = (const bf16_t*)W; p.ldw = ldw; p.bias = (const float*)bias; p.out = out; p.ldo = ldo;
   p.M = M; p.N = N; p.K = K;
+  p.cs = nullptr; p.slot = nullptr;
+  p.q_out = nullptr; p.kc = nullptr; p.vc = nullptr; p.nq = p.nkv = p.hd = p.ps = 0; p.pair_tiles = 0;
   // as many rounds of tiles as 16-row tiles need, with rows per tile cut down to what fills them evenly
   p.rows = 16;
   if (epilogue != EPI_SWIGLU) {
@@ -260,5 +335,50 @@ extern "C" int qvl_gemm_resident(const void* x, int ldx, const void* h, int ldh,
   else if (epilogue == EPI_SWIGLU) QVL_RES(bf16_t, EPI_SWIGLU);
   else return QVL_ERR_DTYPE;
 #undef QVL_RES
+  return qvl_launch_status();
+}
+
+// The stacked query | key | value projection of at most 16 tokens with rotation and cache write
+// folded in (EPI_ROPE).  x / h / norm_w / eps as in qvl_gemm_resident.  W: [(nq + 2 nkv) hd, K];
+// bias: float32 [(nq + 2 nkv) hd] or null.  cs: float32 [M, hd / 2, 2], cosine and sine of every
+// token's angle at every frequency (1 and 0 where a frequency is not rotated);
+// slot: int32 [M] flat cache slot of each token (null with nkv == 0: queries only);
+// q_out: bfloat16 [M, nq hd]; kc: [pages, nkv, ps, hd]; vc: [pages, nkv, hd, ps].
+// hd must be a multiple of 16 (the rotation covers the whole head, channel f with f + hd / 2).
+extern "C" int qvl_gemm_resident_rope(const void* x, int ldx, const void* h, int ldh, const void* norm_w, float eps,
+                                      const void* W, int ldw, const void* bias, int M, int K, const void* cs,
+                                      const void* slot, void* q_out, void* kc, void* vc, int nq, int nkv, int hd, int ps,
+                                      int max_blocks, hipStream_t stream) {
+  if (M <= 0) return QVL_OK;
+  if (M > 16) return QVL_ERR_LIMIT;
+  if (K <= 0 || K % 8 || ldw % 8 || ldw < K || max_blocks <= 0 || !W || !q_out) return QVL_ERR_SHAPE;
+  if (nq <= 0 || nkv < 0 || hd <= 0 || hd % 16 || ps <= 0 || !cs) return QVL_ERR_SHAPE;
+  if (nkv > 0 && (!slot || !kc || !vc)) return QVL_ERR_SHAPE;
+  const bool norm = h != nullptr;
+  if (norm) {
+    if (x || !norm_w || K > PASS_K || ldh % 4 || ldh < K) return QVL_ERR_SHAPE;
+  } else if (!x || ldx % 8 || ldx < K) {
+    return QVL_ERR_SHAPE;
+  }
+  ResidentArgs p;
+  p.X = (const bf16_t*)x; p.ldx = ldx; p.H = (const float*)h; p.ldh = ldh; p.norm_w = (const float*)norm_w;
+  p.eps = eps; p.W = (const bf16_t*)W; p.ldw = ldw; p.bias = (const float*)bias; p.out = nullptr; p.ldo = 0;
+  p.M = M; p.N = (nq + 2 * nkv) * hd; p.K = K;
+  // query and key heads in tiles of 8 + 8 rows, then the value rows in tiles as small as fills
+  // the compute units evenly (36 heads of 128 on 256 units: 256 tiles of 16 and 256 of 2)
+  p.pair_tiles = (nq + nkv) * (hd / 16);
+  p.rows = 16;
+  int value_tiles = 0;
+  if (nkv > 0) {
+    const long long vrows = (long long)nkv * hd, per_round = 16LL * max_blocks;
+    const long long rounds = (vrows + per_round - 1) / per_round;
+    p.rows = (int)((vrows + rounds * max_blocks - 1) / (rounds * max_blocks));
+    value_tiles = (int)((vrows + p.rows - 1) / p.rows);
+  }
+  p.ntiles = p.pair_tiles + value_tiles;
+  p.cs = (const float*)cs; p.slot = (const int*)slot; p.q_out = (bf16_t*)q_out; p.kc = (bf16_t*)kc;
+  p.vc = (bf16_t*)vc; p.nq = nq; p.nkv = nkv; p.hd = hd; p.ps = ps;
+  if (norm) launch<bf16_t, PRO_NORM, EPI_ROPE>(p, max_blocks, stream);
+  else launch<bf16_t, PRO_PLAIN, EPI_ROPE>(p, max_blocks, stream);
   return qvl_launch_status();
 }

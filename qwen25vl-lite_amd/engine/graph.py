@@ -123,8 +123,10 @@ class _Graph:
             # then once more under capture; a decode step only writes the step's own cache slots
             # and the logits, so running it again with the same inputs changes nothing
             for _ in range(2):
+                self.step.per_pass.clear()
                 runner.model.forward(self.step, runner.slots)
             torch.cuda.synchronize()
+            self.step.per_pass.clear()    # what a pass computes from the step's values is computed in the graph
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 self.logits = runner.model.forward(self.step, runner.slots)

@@ -14,7 +14,7 @@ import torch
 
 from .library import load_library
 
-__all__ = [
+__all__ = ["rope_table", 
     "KernelError", "embed_gather", "add_rmsnorm", "rope_kv_write", "paged_attention_generic", "swiglu",
     "gemm_f32", "dtype_code",
 ]
@@ -168,6 +168,23 @@ def rope_kv_write(x: torch.Tensor, bias: Optional[torch.Tensor], positions: torc
               _ptr(freq_row), _ptr(slots), _ptr(q_out), _ptr(k_cache), _ptr(v_cache), n, nq, nkv, hd, rot_half,
               int(page_size), dtype_code(x.dtype), dtype_code(odt), _stream()), "rope_kv_write")
     return q_out
+
+
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, freq_row: torch.Tensor, n: int) -> torch.Tensor:
+    """Cosine and sine of every token's rotation angle: float32 ``[n, rot/2, 2]`` with
+    ``(cos, sin)(positions[freq_row[f], i] * inv_freq[f])``, or ``(1, 0)`` where ``freq_row[f] < 0``."""
+    _dev(positions, inv_freq, freq_row)
+    rot_half = inv_freq.shape[0]
+    _need(inv_freq.dtype == torch.float32 and inv_freq.is_contiguous(), "inv_freq must be float32 [rot/2]")
+    _need(freq_row.dtype == torch.int32 and freq_row.shape == (rot_half,) and freq_row.is_contiguous(),
+          "freq_row must be int32 [rot/2]")
+    _need(positions.dtype == torch.int32 and positions.dim() == 2 and positions.shape[1] >= n
+          and positions.stride(1) == 1, "positions must be int32 [rows, N]")
+    out = torch.empty((n, rot_half, 2), dtype=torch.float32, device=positions.device)
+    fn = _fn("elementwise", "qvl_rope_table", [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(positions), positions.stride(0), _ptr(inv_freq), _ptr(freq_row), _ptr(out), int(n), rot_half,
+              _stream()), "rope_table")
+    return out
 
 
 def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,

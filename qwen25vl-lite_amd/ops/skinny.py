@@ -14,7 +14,7 @@ import torch
 
 from .kernels import _check, _fn, _ptr, _stream, dtype_code
 
-__all__ = ["resident_product", "takes_resident", "try_streaming", "RESIDENT_ROWS", "RESIDENT_NORM_K", "MAX_ROWS",
+__all__ = ["resident_product", "takes_resident", "qkv_rope_product", "takes_qkv_rope", "try_streaming", "RESIDENT_ROWS", "RESIDENT_NORM_K", "MAX_ROWS",
            "STORE", "RESIDUAL", "SWIGLU"]
 
 MAX_ROWS = 32            # the streaming kernel's limit in use
@@ -81,6 +81,57 @@ def resident_product(weight: torch.Tensor, *, x: Optional[torch.Tensor] = None, 
               _ptr(norm_weight), float(eps), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(out), out.stride(0),
               m, n, k, dtype_code(odt), epilogue, _compute_units(src.device), _stream()), "linear (resident)")
     return out
+
+
+def takes_qkv_rope(m: int, k: int, weight: torch.Tensor, head_dim: int, rot_half: int, cache_dtype, *,
+                   norm: bool = False) -> bool:
+    """Whether the resident kernel can rotate and store the stacked projection by itself: bfloat16,
+    a head size in steps of 16 and a rotation over the whole head."""
+    return (takes_resident(m, k, weight, norm=norm) and head_dim % 16 == 0 and 2 * rot_half == head_dim
+            and cache_dtype in (None, torch.bfloat16))
+
+
+def qkv_rope_product(weight: torch.Tensor, cs: torch.Tensor, *, x: Optional[torch.Tensor] = None,
+                     h: Optional[torch.Tensor] = None, norm_weight: Optional[torch.Tensor] = None, eps: float = 0.0,
+                     bias: Optional[torch.Tensor] = None, slots: Optional[torch.Tensor] = None,
+                     k_cache: Optional[torch.Tensor] = None, v_cache: Optional[torch.Tensor] = None,
+                     num_q_heads: int, num_kv_heads: int, head_dim: int, page_size: int) -> torch.Tensor:
+    """The stacked query | key | value projection of at most 16 tokens with the rotation and the
+    cache write inside the product's kernel: returns the rotated queries ``[M, nq hd]`` (bfloat16);
+    rotated keys and values are in their page slots.  ``cs`` is :func:`kernels.rope_table` of the
+    step's tokens.  With ``num_kv_heads == 0`` the weight holds query rows only."""
+    src = x if x is not None else h
+    m, k = src.shape
+    nq, nkv, hd = int(num_q_heads), int(num_kv_heads), int(head_dim)
+    if weight.shape != ((nq + 2 * nkv) * hd, k) or not takes_qkv_rope(m, k, weight, hd, cs.shape[1], None,
+                                                                        norm=h is not None):
+        raise ValueError("the resident kernel does not take this projection")
+    if x is not None and (x.dtype != torch.bfloat16 or not _rows_aligned(x, 8)):
+        raise ValueError("x must be bfloat16 with 16-byte aligned rows")
+    if h is not None and (h.dtype != torch.float32 or not _rows_aligned(h, 4) or norm_weight is None
+                          or norm_weight.dtype != torch.float32 or norm_weight.shape != (k,)):
+        raise ValueError("h must be float32 rows with a float32 norm weight of their width")
+    if bias is not None and (bias.dtype != torch.float32 or not bias.is_contiguous() or bias.shape != (weight.shape[0],)):
+        raise ValueError("bias must be float32 [(nq + 2 nkv) hd]")
+    if cs.dtype != torch.float32 or cs.shape != (m, hd // 2, 2) or not cs.is_contiguous():
+        raise ValueError("cs must be float32 [M, hd/2, 2]")
+    if nkv:
+        if (slots is None or slots.dtype != torch.int32 or slots.shape != (m,) or not slots.is_contiguous()
+                or k_cache is None or v_cache is None or k_cache.dtype != torch.bfloat16
+                or v_cache.dtype != torch.bfloat16 or not k_cache.is_contiguous() or not v_cache.is_contiguous()
+                or tuple(k_cache.shape[1:]) != (nkv, page_size, hd) or tuple(v_cache.shape[1:]) != (nkv, hd, page_size)
+                or v_cache.shape[0] != k_cache.shape[0]):
+            raise ValueError("slots int32 [M] and bfloat16 caches [pages, nkv, ps, hd] / [pages, nkv, hd, ps] are needed")
+    q_out = torch.empty((m, nq * hd), dtype=torch.bfloat16, device=src.device)
+    fn = _fn("gemm_resident", "qvl_gemm_resident_rope",
+             [_c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_float, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr,
+              _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(x), x.stride(0) if x is not None else 0, _ptr(h), h.stride(0) if h is not None else 0,
+              _ptr(norm_weight), float(eps), _ptr(weight), weight.stride(0), _ptr(bias), m, k, _ptr(cs),
+              _ptr(slots if nkv else None), _ptr(q_out), _ptr(k_cache if nkv else None),
+              _ptr(v_cache if nkv else None), nq, nkv, hd, int(page_size), _compute_units(src.device), _stream()),
+           "linear (resident, rotation and cache write)")
+    return q_out
 
 
 def prefers_streaming(m: int, n: int, k: int) -> bool:

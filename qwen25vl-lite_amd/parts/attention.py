@@ -12,9 +12,9 @@ from typing import Dict, Optional
 
 import torch
 
-from ..ops import kernels
+from ..ops import kernels, skinny
 from ..ops.attention import paged_attention
-from ..ops.linear import linear, linear_into
+from ..ops.linear import NormedRows, linear, linear_into
 from .base import (CacheNeed, LayerSlot, Mixer, ParamSpec, PartSpec, StepContext, build_part, register_part)
 
 __all__ = ["PagedAttention"]
@@ -93,16 +93,43 @@ class PagedAttention(Mixer):
         if slot.writes == self.kv_shared:
             raise RuntimeError("a layer without key/value projections must read another layer's cache, "
                                "and a layer with them must write its own")
+        inv_freq, freq_row = self.position.rotary_tables(self.hd)
+        q = self._project_few_rows(x, step, group, slot, write, inv_freq, freq_row)
+        if q is None:
+            q = self._project(x, step, group, slot, write, inv_freq, freq_row)
+        o = paged_attention(q, slot.k_cache, slot.v_cache, group.block_table, step, self.nq, self.window, self.scale)
+        return linear_into(step.residual, o, self.w_out)
+
+    def _project(self, x, step, group, slot, write, inv_freq, freq_row) -> torch.Tensor:
         # Projections are written out in float32 (the accumulator, unrounded): bias, rotation and
         # the residual sum then happen in float32 and each stored value is rounded once.
         qkv = linear(x, self.w_in, out_dtype=torch.float32)
-        inv_freq, freq_row = self.position.rotary_tables(self.hd)
-        q = kernels.rope_kv_write(
+        return kernels.rope_kv_write(
             qkv, self.b_in, step.positions, inv_freq, freq_row,
             group.slot_mapping if write else None, slot.k_cache if write else None, slot.v_cache if write else None,
             self.nq, self.nkv if write else 0, self.hd, group.page_size, out_dtype=self.dtype)
-        o = paged_attention(q, slot.k_cache, slot.v_cache, group.block_table, step, self.nq, self.window, self.scale)
-        return linear_into(step.residual, o, self.w_out)
+
+    def _project_few_rows(self, x, step, group, slot, write, inv_freq, freq_row) -> Optional[torch.Tensor]:
+        """A decode step's few bfloat16 rows: projection, bias, rotation and cache write in one
+        kernel (the float32 sums never leave it).  The cosines and sines of the step's angles are
+        computed once per step and position encoding, by the first layer that needs them."""
+        lazy = isinstance(x, NormedRows)
+        m, k = x.shape
+        if self.dtype != torch.bfloat16 or not skinny.takes_qkv_rope(
+                m, k, self.w_in, self.hd, inv_freq.shape[0], slot.k_cache.dtype if write else None, norm=lazy):
+            return None
+        if not lazy and (x.dtype != torch.bfloat16 or x.stride(1) != 1 or x.stride(0) % 8 or x.data_ptr() % 16):
+            return None
+        key = ("rope_cs", self.position.table_key(self.hd))
+        cs = step.per_pass.get(key)
+        if cs is None:
+            cs = step.per_pass[key] = kernels.rope_table(step.positions, inv_freq, freq_row, m)
+        src = dict(h=x.h, norm_weight=x.weight, eps=x.eps) if lazy else dict(x=x)
+        return skinny.qkv_rope_product(
+            self.w_in, cs, bias=self.b_in, slots=group.slot_mapping if write else None,
+            k_cache=slot.k_cache if write else None, v_cache=slot.v_cache if write else None,
+            num_q_heads=self.nq, num_kv_heads=self.nkv if write else 0, head_dim=self.hd,
+            page_size=group.page_size, **src)
 
 
 register_part("mixer", "paged_attention", PagedAttention)

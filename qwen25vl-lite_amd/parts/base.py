@@ -118,6 +118,9 @@ class StepContext:
     dtype: torch.dtype = torch.float32
     residual: Optional[torch.Tensor] = None   # set by a block while a part may add its result in place
     derived: Dict[Any, Any] = field(default_factory=dict)   # per-step arrays kernels derive once (tile lists)
+    # tensors computed from the step's values once per forward pass (rotation tables): a context
+    # that is run again with new values (a captured step) starts each pass with this empty
+    per_pass: Dict[Any, Any] = field(default_factory=dict)
 
 
 @dataclass
@@ -180,6 +183,11 @@ class PositionEncoding(Part):
     def rotary_tables(self, head_dim: int) -> Tuple[torch.Tensor, torch.Tensor]:
         """``(inv_freq float32 [rot/2], freq_row int32 [rot/2])`` on the device."""
         raise NotImplementedError
+
+    def table_key(self, head_dim: int):
+        """A hashable value that is equal for encodings with equal tables: layers whose encodings
+        agree share what a step derives from the tables.  Default: this instance only."""
+        return (id(self), head_dim)
 
 
 class Block(Part):

@@ -43,6 +43,9 @@ class MRoPE(PositionEncoding):
             raise ValueError("MRoPE takes three section counts (t, h, w)")
         self._tables = {}
 
+    def table_key(self, head_dim: int):
+        return ("mrope", self.theta, self.sections, head_dim)
+
     def rotary_tables(self, head_dim: int) -> Tuple[torch.Tensor, torch.Tensor]:
         if head_dim not in self._tables:
             half = head_dim // 2
@@ -71,6 +74,9 @@ class RoPE1D(PositionEncoding):
         self.theta = float(params["theta"])
         self.rotary_dim = params.get("rotary_dim")
         self._tables = {}
+
+    def table_key(self, head_dim: int):
+        return ("rope", self.theta, self.rotary_dim, head_dim)
 
     def rotary_tables(self, head_dim: int) -> Tuple[torch.Tensor, torch.Tensor]:
         if head_dim not in self._tables:

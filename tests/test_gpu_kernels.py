@@ -338,3 +338,53 @@ def test_no_cpu_path():
         linear(torch.zeros(2, 4), torch.zeros(3, 4))
     with pytest.raises(kernels.KernelError):
         kernels.swiglu(torch.zeros(2, 4, dtype=torch.float16).cuda())
+
+
+@pytest.mark.parametrize("m, nq, nkv, hd, k, bias, lazy", [(1, 4, 2, 16, 64, True, False), (8, 28, 4, 128, 3584, True, True),
+                                                         (16, 6, 3, 48, 136, False, True), (5, 3, 0, 80, 104, True, False)])
+def test_projection_with_rotation_and_cache_write_folded_in(m, nq, nkv, hd, k, bias, lazy):
+    """The stacked q | k | v projection of a few rows that rotates and stores inside the product's
+    kernel equals the product followed by the rotation kernel: queries, and every slot of the
+    cache (the slots of other tokens keep their stale values)."""
+    from qwen25vl_lite_amd.ops import kernels, skinny
+    from qwen25vl_lite_amd.ops.linear import linear
+    torch.manual_seed(hd + m)
+    ps, pages = 16, 7
+    n_out = (nq + 2 * nkv) * hd
+    w = (torch.randn(n_out, k) / math.sqrt(k)).bfloat16().cuda()
+    b = torch.randn(n_out).cuda() if bias else None
+    h = (torch.randn(m, k) * 2).cuda()
+    g = (1 + 0.1 * torch.randn(k)).cuda()
+    x = kernels.add_rmsnorm(h, None, g, 1e-6, torch.bfloat16)
+    half = hd // 2
+    inv_freq = (1.0 / (10000.0 ** (torch.arange(0, hd, 2, dtype=torch.float32) / hd))).cuda()
+    freq_row = (torch.arange(half) % 3).int().cuda()
+    if half > 3:
+        freq_row[3] = -1                        # a frequency that is not rotated
+    pos = torch.randint(0, 40000, (3, m), dtype=torch.int32).cuda()
+    slots = torch.randperm(pages * ps)[:m].int().cuda()
+    if m > 2:
+        slots[1] = -1                           # a token without a slot writes nothing
+    kc0 = torch.randn(pages, max(nkv, 1), ps, hd).bfloat16().cuda()
+    vc0 = torch.randn(pages, max(nkv, 1), hd, ps).bfloat16().cuda()
+    kc_a, vc_a, kc_b, vc_b = kc0.clone(), vc0.clone(), kc0.clone(), vc0.clone()
+    qkv = linear(x, w, out_dtype=torch.float32)
+    q_a = kernels.rope_kv_write(qkv, b, pos, inv_freq, freq_row, slots if nkv else None, kc_a if nkv else None,
+                                vc_a if nkv else None, nq, nkv, hd, ps, out_dtype=torch.bfloat16)
+    assert skinny.takes_qkv_rope(m, k, w, hd, half, torch.bfloat16, norm=lazy)
+    cs = kernels.rope_table(pos, inv_freq, freq_row, m)
+    src = dict(h=h, norm_weight=g, eps=1e-6) if lazy else dict(x=x)
+    q_b = skinny.qkv_rope_product(w, cs, bias=b, slots=slots if nkv else None, k_cache=kc_b if nkv else None,
+                                  v_cache=vc_b if nkv else None, num_q_heads=nq, num_kv_heads=nkv, head_dim=hd,
+                                  page_size=ps, **src)
+    tol = dict(atol=2e-2, rtol=2e-2)           # one bfloat16 rounding of values of a few units
+    assert torch.allclose(q_b.float(), q_a.float(), **tol), (q_b.float() - q_a.float()).abs().max()
+    assert torch.allclose(kc_b.float(), kc_a.float(), **tol) and torch.allclose(vc_b.float(), vc_a.float(), **tol)
+    if nkv:   # something was written, and only in the tokens' slots
+        assert not torch.equal(kc_b, kc0) and not torch.equal(vc_b, vc0)
+        touched = (kc_b != kc0).any(dim=3).any(dim=1).flatten().nonzero().flatten().tolist()
+        assert set(touched) <= set(s for s in slots.tolist() if s >= 0)
+    # a head size whose rotation the kernel does not take, or a cache of another type, is refused
+    assert not skinny.takes_qkv_rope(m, k, w, 24, 12, torch.bfloat16)
+    assert not skinny.takes_qkv_rope(m, k, w, hd, half - 1, torch.bfloat16)
+    assert not skinny.takes_qkv_rope(m, k, w, hd, half, torch.float32)
