@@ -637,7 +637,7 @@ __global__ __launch_bounds__(64 * BLK_WAVES, BLK_PER_CU) void attn_mfma_block_ke
 #define PART_COLS (HD + 4)
 #define PART_STRIDE (16 * PART_COLS)
 #if HD <= 128
-#define COOP_WAVES 4
+#define COOP_WAVES 8
 #else
 #define COOP_WAVES 2
 #endif
