@@ -77,7 +77,7 @@ __device__ __forceinline__ uint32_t pack2(float a, float b) {
 
 template <typename TO, int PRO, int EPI, bool ONE_PASS>
 __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) {
-  __shared__ float red[RW][256];
+  __shared__ float red[2][RW][256];   // two buffers: a tile's sums are read while the next tile's are written
   __shared__ float rowsq[RW][16];
   __shared__ __attribute__((aligned(16))) float gains[PRO == PRO_NORM ? RW : 1][RK * 32];   // norm weights of each wave's columns
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lg = lane >> 4, r = lane & 15;
@@ -196,16 +196,21 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
     return e;
   };
   // ---- merge the waves' sums of one tile and write the result -----------------------------------
+  // One barrier per tile: the sums go into the buffer that was read two tiles ago; whoever reads
+  // it (the first four waves) has passed the barrier of the tile in between since.
+  int parity = 0;
   auto finish = [&](int tile, const f32x4_t& acc, const Epi& epi) {
+    float (*buf)[256] = red[parity];
+    parity ^= 1;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) red[wave][(4 * lg + i) * 16 + r] = acc[i];
+    for (int i = 0; i < 4; ++i) buf[wave][(4 * lg + i) * 16 + r] = acc[i];
     __syncthreads();
     if (threadIdx.x < 256) {
       const int e = threadIdx.x;
       const int m = e >> 4, nl = e & 15, n = w_row(tile, nl);
       float sum = 0.f;
 #pragma unroll
-      for (int w = 0; w < RW; ++w) sum += red[w][nl * 16 + m];
+      for (int w = 0; w < RW; ++w) sum += buf[w][nl * 16 + m];
       if (EPI == EPI_SWIGLU) {
         const float up = __shfl_down(sum, 8, QVL_WAVE);  // rows 8..15 of the tile are the up rows
         if (nl < 8 && m < p.M && n < p.N) {
@@ -240,7 +245,6 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
         }
       }
     }
-    __syncthreads();
   };
   auto product = [&](const bf16x8_t* a, const bf16x8_t* xb, f32x4_t acc) {
 #pragma unroll
