@@ -27,15 +27,24 @@ HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 MFMA_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
 
 
-def seven_b_config(layers=None):
-    """configs[2] of BASELINE.json as a config.json dictionary."""
+SIZES = {   # layer sizes of BASELINE.json's configs[3], [2] and [4]
+    "3b": dict(hidden_size=2048, intermediate_size=11008, num_hidden_layers=36, num_attention_heads=16,
+               num_key_value_heads=2, vocab_size=151936, tie_word_embeddings=True),
+    "7b": dict(hidden_size=3584, intermediate_size=18944, num_hidden_layers=28, num_attention_heads=28,
+               num_key_value_heads=4, vocab_size=152064, tie_word_embeddings=False),
+    "72b": dict(hidden_size=8192, intermediate_size=29568, num_hidden_layers=80, num_attention_heads=64,
+                num_key_value_heads=8, vocab_size=152064, tie_word_embeddings=False),
+}
+
+
+def seven_b_config(layers=None, size="7b"):
+    """configs[2] of BASELINE.json (or another of its sizes) as a config.json dictionary."""
     raw = {
         "architectures": ["Qwen2_5_VLForConditionalGeneration"], "model_type": "qwen2_5_vl",
-        "tie_word_embeddings": False, "hidden_size": 3584, "intermediate_size": 18944,
-        "num_hidden_layers": 28, "num_attention_heads": 28, "num_key_value_heads": 4, "vocab_size": 152064,
         "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "sliding_window": 32768, "use_sliding_window": False,
         "max_position_embeddings": 8192, "rope_scaling": {"type": "mrope", "mrope_section": [16, 24, 24]},
     }
+    raw.update(SIZES[size])
     if layers:
         raw["num_hidden_layers"] = int(layers)
     return raw
@@ -70,9 +79,13 @@ def main(argv=None) -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--prompt-tokens", type=int, default=512)
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration has")
+    ap.add_argument("--size", default="7b", choices=sorted(SIZES), help="layer sizes (default: the 7B decoder)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and the prefill")
     ap.add_argument("--prefill-only", action="store_true", help="only the 2,048-token prefill (for profiles)")
+    ap.add_argument("--serving", action="store_true",
+                    help="instead: continuous batching of 64 requests (BASELINE.json configs[3]'s workload: prompts "
+                         "of 64 to 2048 tokens, 32 to 512 generated, a quarter sharing a 1024-token prefix)")
     ap.add_argument("--no-graph", action="store_true", help="do not replay decode steps from a HIP graph")
     ap.add_argument("--no-tune", action="store_true", help="do not let TunableOp choose the library's kernels")
     args = ap.parse_args(argv)
@@ -86,7 +99,7 @@ def main(argv=None) -> int:
     from qwen25vl_lite_amd.config import dtype_from_name
     from qwen25vl_lite_amd.weights import fill_random
 
-    cfg = Qwen25VLConfig.from_dict(seven_b_config(args.layers))
+    cfg = Qwen25VLConfig.from_dict(seven_b_config(args.layers, args.size))
     t = cfg.text_config
     dtype = dtype_from_name(args.dtype)
     model = build_model(cfg, dtype, "cuda:0")
@@ -152,6 +165,44 @@ def main(argv=None) -> int:
         torch.cuda.empty_cache()
         return min(times)
 
+    if args.serving:
+        import random
+        rng = random.Random(0)
+        shared = prompt(1024)
+        reqs = []
+        for i in range(64):
+            n, out = rng.randint(64, 2048), rng.randint(32, 512)
+            toks = (shared + prompt(max(0, n - 1024)))[:max(n, 1025)] if i % 4 == 0 else prompt(n)
+            reqs.append((toks, out))
+        need_pages = sum((len(tk) + out + page - 1) // page + 1 for tk, out in reqs)
+        ecfg = EngineConfig(num_blocks=need_pages, block_size=page, max_num_seqs=64, max_num_batched_tokens=4096,
+                            max_model_len=max_ctx, enable_prefix_cache=True, dtype=dtype, device="cuda:0",
+                            hip_graph=not args.no_graph, tune_library_products=not args.no_tune)
+
+        def serve():
+            runner = ModelRunner(model, ecfg)
+            engine = LLMEngine(runner, ecfg)
+            for tk, out in reqs:
+                engine.add_request(tk, SamplingParams(temperature=0.0, max_tokens=out, ignore_eos=True))
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            outs = engine.run_until_complete()
+            torch.cuda.synchronize()
+            return time.perf_counter() - t0, outs, engine.stats()
+
+        serve()                                   # library tuning, kernel builds, first graph captures
+        sec, outs, stats = serve()
+        generated = sum(len(o.output_token_ids) for o in outs)
+        prompt_tokens = sum(len(tk) for tk, _ in reqs)
+        print(json.dumps({
+            "metric": f"continuous batching, generated tok/s (Qwen2.5-VL-{args.size.upper()} text decoder sizes, "
+                      f"{args.dtype}, 64 requests)",
+            "value": round(generated / sec, 1), "unit": "tokens/s", "seconds": round(sec, 3),
+            "generated_tokens": generated, "prompt_tokens": prompt_tokens, "steps": int(stats["steps"]),
+            "prefix_cache_hits": int(stats["prefix_cache_hits"]),
+            "prefix_cache_tokens_saved": int(stats["prefix_cache_tokens_saved"]),
+            "preemptions": int(stats["preemptions"]), "data": "synthetic"}))
+        return 0
     if args.prefill_only:
         sec = prefill_rate(2048)
         print(json.dumps({"prefill": {"value": round(2048 / sec, 1), "tokens": 2048, "ms": round(sec * 1e3, 3)}}))
@@ -161,13 +212,14 @@ def main(argv=None) -> int:
     achieved = need / (ms_per_step * 1e-3) / 1e9
     peak_key = "bf16" if args.dtype == "bfloat16" else "fp32"
     line = {
-        "metric": "decode tok/s (Qwen2.5-VL-7B text decoder, bf16, batch 8, 512-token prompts)",
+        "metric": f"decode tok/s (Qwen2.5-VL-{args.size.upper()} text decoder, {args.dtype}, batch {args.batch}, "
+                  f"{args.prompt_tokens}-token prompts)",
         "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
         "config": {
-            "model": "Qwen2.5-VL-7B text decoder (random weights)", "layers": t.num_hidden_layers,
-            "layers_of_config": 28, "hidden_size": t.hidden_size, "heads": t.num_attention_heads,
+            "model": f"Qwen2.5-VL-{args.size.upper()} text decoder (random weights)", "layers": t.num_hidden_layers,
+            "layers_of_config": SIZES[args.size]["num_hidden_layers"], "hidden_size": t.hidden_size, "heads": t.num_attention_heads,
             "kv_heads": t.num_key_value_heads, "head_dim": t.head_dim, "intermediate_size": t.intermediate_size,
             "vocab_size": t.vocab_size, "global_batch": args.batch, "seq_len": args.prompt_tokens,
             "context_mid": ctx_mid, "max_context": max_ctx, "page_size": page, "parallelism": "single GPU",

@@ -33,7 +33,8 @@ __global__ void attn_generic_kernel(const T* __restrict__ q, const T* __restrict
     const bool valid = j >= lo && j <= p;
     float s = -INFINITY;
     if (valid) {
-      const size_t page = (size_t)bt[j / ps];
+      const int pk = bt[j / ps];
+      const size_t page = (size_t)(pk < 0 ? 0 : pk);   // a table without this page: read page 0, never out of bounds
       const T* kr = kc + ((page * nkv + kvh) * ps + (size_t)(j % ps)) * hd;
       float dot = 0.f;
       for (int d = 0; d < hd; ++d) dot += sq[d] * ldf<T>(kr + d);
@@ -50,7 +51,8 @@ __global__ void attn_generic_kernel(const T* __restrict__ q, const T* __restrict
       const float pv = __shfl(pj, jj, QVL_WAVE);
       const int ja = c * 64 + jj;
       if (ja < lo) continue;
-      const size_t page = (size_t)bt[ja / ps];
+      const int pv_page = bt[ja / ps];
+      const size_t page = (size_t)(pv_page < 0 ? 0 : pv_page);
       const T* vr = vc + ((page * nkv + kvh) * hd) * ps + (size_t)(ja % ps);
 #pragma unroll
       for (int i = 0; i < ATTN_MAX_HD / 64; ++i) {

@@ -4,9 +4,15 @@ A decode step of a 7B model is a few hundred short kernels; launched one by one 
 the host, not the GPU, sets the step time (the reference measured the same on its hardware,
 reference src/qwen25vl_lite/graphs.py:3-7, and also answers with graph capture).  A step in
 which every request brings exactly one token has a fixed shape, so it is captured once per
-(batch size, context bucket) and replayed: per step the host fills one pinned buffer with the
+(batch bucket, context bucket) and replayed: per step the host fills one pinned buffer with the
 step's integers (token ids, positions, page slots, block tables, context lengths), copies it to
 a fixed device buffer in one transfer, and launches the graph.
+
+Batch sizes are rounded up to 1, 2, 3, 4, 6, 8, 12, 16, ... so that a server whose batch shrinks
+and grows request by request captures a dozen graphs, not one per size.  The rows added are
+padding: token 0 at position 0 with a context of one key, no page slot to write to (slot -1), a
+block table that names page 0 for that key (whatever it holds is finite) and the spare state
+row; their logits are computed and dropped.
 
 The context bucket (the next power of two above the longest context) only fixes how many waves
 the attention kernel splits a request's keys over; the true lengths travel in the buffer.
@@ -23,6 +29,16 @@ from ..parts.base import GroupStep, StepContext
 from .batch import StepEntry
 
 __all__ = ["DecodeGraphs"]
+
+
+def _batch_bucket(n: int, most: int) -> int:
+    """The smallest of 1, 2, 3, 4, 6, 8, 12, 16, 24, ... that holds n rows (at most ``most``)."""
+    b = 1
+    while True:
+        for cand in (b, b + b // 2):
+            if cand >= n:
+                return min(cand, max(most, n))
+        b *= 2
 
 
 def _bucket(n: int, floor: int = 256) -> int:
@@ -90,14 +106,21 @@ class _Graph:
 
     def fill(self, entries: Sequence[StepEntry]) -> None:
         cache, ps, h = self.runner.cache, self.ps, self.h
+        n, b = len(entries), self.batch
         self.copied.synchronize()          # the previous transfer has read the pinned buffer
-        starts = np.fromiter((e.start for e in entries), np.int32, self.batch)
-        deltas = np.fromiter((e.rope_delta for e in entries), np.int32, self.batch)
-        h("token_ids")[:] = np.fromiter((e.tokens[0] for e in entries), np.int32, self.batch)
+        starts = np.zeros(b, np.int32)     # rows from n on are padding: position 0, one key, no slot
+        deltas = np.zeros(b, np.int32)
+        starts[:n] = np.fromiter((e.start for e in entries), np.int32, n)
+        deltas[:n] = np.fromiter((e.rope_delta for e in entries), np.int32, n)
+        tokens = h("token_ids")
+        tokens[:n] = np.fromiter((e.tokens[0] for e in entries), np.int32, n)
+        tokens[n:] = 0
         h("token_seqpos")[:] = starts
-        h("positions", (self.rows, self.batch))[:] = starts + deltas
+        h("positions", (self.rows, b))[:] = starts + deltas
         h("ctx_len")[:] = starts + 1
-        h("req_slots")[:] = np.fromiter((cache.slot_of(e.req_id) for e in entries), np.int32, self.batch)
+        slots_of = h("req_slots")
+        slots_of[:n] = np.fromiter((cache.slot_of(e.req_id) for e in entries), np.int32, n)
+        slots_of[n:] = self.runner.pad_state_slot
         for g in range(self.ngroups):
             table_np, lens, slots = self.tables[g], self.row_len[g], h(f"slots{g}")
             for i, e in enumerate(entries):
@@ -110,8 +133,16 @@ class _Graph:
                     table_np[i, lens[i]:len(t)] = t[lens[i]:]
                     lens[i] = len(t)
                 slots[i] = t[e.start // ps] * ps + e.start % ps
+            for i in range(n, b):
+                if self.row_req[i] is not None or table_np[i, 0] != 0:
+                    table_np[i, :] = -1
+                    table_np[i, 0] = 0
+                    lens[i] = 0
+                slots[i] = -1
         for i, e in enumerate(entries):
             self.row_req[i] = cache.requests[e.req_id]
+        for i in range(n, b):
+            self.row_req[i] = None
 
     def run(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         runner = self.runner
@@ -132,11 +163,11 @@ class _Graph:
                 self.logits = runner.model.forward(self.step, runner.slots)
             self.graph = graph
         self.graph.replay()
-        return self.logits
+        return self.logits[:len(entries)]
 
 
 class DecodeGraphs:
-    """The graphs of a runner, keyed by (batch size, context bucket)."""
+    """The graphs of a runner, keyed by (batch bucket, context bucket)."""
 
     def __init__(self, runner, max_graphs: int = 32):
         self.runner = runner
@@ -149,7 +180,7 @@ class DecodeGraphs:
 
     def run(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         ctx = max(e.start for e in entries) + 1
-        key = (len(entries), _bucket(ctx))
+        key = (_batch_bucket(len(entries), self.runner.ecfg.max_num_seqs), _bucket(ctx))
         g = self.graphs.get(key)
         if g is None:
             if len(self.graphs) >= self.max_graphs:

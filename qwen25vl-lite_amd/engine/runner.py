@@ -40,8 +40,11 @@ class ModelRunner:
                                   enable_prefix_cache=engine_cfg.enable_prefix_cache,
                                   max_prefix_nodes=max_prefix_nodes)
         self.storage = KVStorage(groups, engine_cfg.num_blocks, engine_cfg.block_size, self.dtype, self.device)
+        # one state row per request slot, and a spare one that the padding rows of a captured
+        # decode step read and write
+        self.pad_state_slot = engine_cfg.max_num_seqs
         self.states: List[Optional[torch.Tensor]] = [
-            None if need is None else torch.zeros((engine_cfg.max_num_seqs, *need.shape), dtype=need.dtype,
+            None if need is None else torch.zeros((engine_cfg.max_num_seqs + 1, *need.shape), dtype=need.dtype,
                                                   device=self.device)
             for need in model.entry_state
         ]

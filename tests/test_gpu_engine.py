@@ -83,6 +83,28 @@ def test_decode_from_hip_graphs_gives_the_same_tokens(model_dirs, name, dtype):
             assert out.output_token_ids == _plain_greedy(d, prompt, p.max_tokens)
 
 
+@pytest.mark.parametrize("name, dtype", [("B_sharp", "float32"), ("C_sharp", "bfloat16")])
+def test_decode_graphs_with_padding_rows(model_dirs, name, dtype):
+    """Batch sizes between the captured ones (7 and 5 requests run in graphs of 8 and 6 rows): the
+    padding rows change nothing for the real ones, and the windowed layers' pages still come back."""
+    from qwen25vl_lite_amd import LLM, SamplingParams
+
+    d = model_dirs[name]
+    vocab = {"B": 509, "C": 300}[name[0]]
+    prompts = [random_tokens(n, vocab, 70 + n) for n in (9, 40, 3, 66, 21, 14, 50)]
+    params = [SamplingParams(temperature=0.0, max_tokens=m, ignore_eos=True) for m in (30, 12, 44, 20, 52, 36, 25)]
+    common = dict(dtype=dtype, num_blocks=96, block_size=16, max_num_seqs=8, max_num_batched_tokens=256,
+                  enable_prefix_cache=False)
+    eager = LLM(d, **common).generate(prompts, params)
+    llm = LLM(d, hip_graph=True, **common)
+    graphed = llm.generate(prompts, params)
+    sizes = sorted({k[0] for k in llm.runner.graphs.graphs})
+    assert 8 in sizes and 6 in sizes and 7 not in sizes and 5 not in sizes, sizes
+    for a, b in zip(eager, graphed):
+        assert a.output_token_ids == b.output_token_ids
+    assert llm.runner.cache.pages_in_use() == [0] * len(llm.runner.cache.groups)
+
+
 def test_prefix_reuse_gives_the_same_tokens(model_dirs):
     # reference tests/test_chunked_prefill.py:193-227, tests/test_engine.py:57-106
     from qwen25vl_lite_amd import LLM, SamplingParams
