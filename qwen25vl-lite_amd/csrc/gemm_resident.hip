@@ -61,6 +61,10 @@ struct ResidentArgs {
   bf16_t* vc;            // [pages, nkv, hd, ps]
   int nq, nkv, hd, ps;
   int pair_tiles;        // tiles of query and key heads (16 rows each); value tiles of `rows` rows follow
+  // EPI_SWIGLU: the first whole_tiles tiles are whole groups of 8 + 8 rows; each group after them
+  // is cut into `parts` tiles of `pairs` gate rows and their up rows, so that the last round of
+  // tiles is as even as the rounds before it
+  int whole_tiles, parts, pairs;
 };
 
 __device__ __forceinline__ bf16x8_t load8(const bf16_t* p) {
@@ -157,11 +161,16 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
       }
       return (p.nq + p.nkv) * p.hd + (tile - p.pair_tiles) * p.rows + i;   // value rows
     }
+    if (EPI == EPI_SWIGLU && tile >= p.whole_tiles) {
+      // a part of one of the last groups: `pairs` gate rows and the up rows that belong to them
+      const int part = tile - p.whole_tiles, group = p.whole_tiles + part / p.parts, s = part % p.parts;
+      return (i & 7) < p.pairs ? group * 16 + (i >> 3) * 8 + s * p.pairs + (i & 7) : -1;
+    }
     return tile * p.rows + i;
   };
   auto load_w = [&](int tile, int k0, bf16x8_t* a) {
     const int row = w_row(tile, r);
-    const bool row_ok = r < tile_rows(tile) && row < p.N;
+    const bool row_ok = r < tile_rows(tile) && row >= 0 && row < p.N;
     const bf16_t* wrow = p.W + (size_t)(row_ok ? row : 0) * p.ldw;
 #pragma unroll
     for (int u = 0; u < RK; ++u) {
@@ -213,9 +222,9 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
       for (int w = 0; w < RW; ++w) sum += buf[w][nl * 16 + m];
       if (EPI == EPI_SWIGLU) {
         const float up = __shfl_down(sum, 8, QVL_WAVE);  // rows 8..15 of the tile are the up rows
-        if (nl < 8 && m < p.M && n < p.N) {
+        if (nl < 8 && m < p.M && n >= 0 && n < p.N) {
           bf16_t* o = reinterpret_cast<bf16_t*>(p.out);
-          o[(size_t)m * p.ldo + tile * 8 + nl] = f32_to_bf16((sum / (1.0f + expf(-sum))) * up);
+          o[(size_t)m * p.ldo + (n >> 4) * 8 + (n & 7)] = f32_to_bf16((sum / (1.0f + expf(-sum))) * up);
         }
       } else if (EPI == EPI_ROPE) {
         sum += epi.bias;
@@ -328,6 +337,16 @@ extern "C" int qvl_gemm_resident(const void* x, int ldx, const void* h, int ldh,
     p.rows = (int)((N + rounds * max_blocks - 1) / (rounds * max_blocks));
   }
   p.ntiles = (N + p.rows - 1) / p.rows;
+  p.whole_tiles = p.ntiles; p.parts = 1; p.pairs = 8;
+  if (epilogue == EPI_SWIGLU) {
+    const int groups = N / 16, left = groups % max_blocks;
+    if (groups > max_blocks && left > 0) {
+      while (p.parts < 8 && left * p.parts * 2 <= max_blocks) p.parts *= 2;
+      p.pairs = 8 / p.parts;
+      p.whole_tiles = groups - left;
+      p.ntiles = p.whole_tiles + left * p.parts;
+    }
+  }
 #define QVL_RES(TO, EPI)                                                    \
   do {                                                                      \
     if (norm) launch<TO, PRO_NORM, EPI>(p, max_blocks, stream);             \
@@ -382,6 +401,7 @@ extern "C" int qvl_gemm_resident_rope(const void* x, int ldx, const void* h, int
   p.ntiles = p.pair_tiles + value_tiles;
   p.cs = (const float*)cs; p.slot = (const int*)slot; p.q_out = (bf16_t*)q_out; p.kc = (bf16_t*)kc;
   p.vc = (bf16_t*)vc; p.nq = nq; p.nkv = nkv; p.hd = hd; p.ps = ps;
+  p.whole_tiles = 0; p.parts = 1; p.pairs = 8;
   if (norm) launch<bf16_t, PRO_NORM, EPI_ROPE>(p, max_blocks, stream);
   else launch<bf16_t, PRO_PLAIN, EPI_ROPE>(p, max_blocks, stream);
   return qvl_launch_status();

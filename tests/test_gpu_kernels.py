@@ -310,7 +310,8 @@ def test_product_added_into_the_residual(m, n, k):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("m, inter, k", [(1, 352, 144), (8, 18944, 3584), (16, 40, 4104), (50, 352, 144)])
+@pytest.mark.parametrize("m, inter, k", [(1, 352, 144), (8, 18944, 3584), (16, 40, 4104), (50, 352, 144),
+                                         (4, 2072, 64), (3, 5136, 72), (2, 8 * 320, 40)])
 def test_gate_up_product_with_the_activation_folded_in(dtype, m, inter, k):
     """Grouped gate | up rows: few bfloat16 rows get silu(gate) * up from the product's own kernel,
     everything else from the product followed by the activation kernel on the grouped columns."""
