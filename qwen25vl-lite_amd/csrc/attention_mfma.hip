@@ -755,7 +755,6 @@ static int check_common(int num_tiles, int nq, int nkv, int ps, int table_width)
   return -1;
 }
 
-extern "C" int qvl_attn_mfma_head_dim() { return HD; }
 // Column tiles per entry of the block list that qvl_attn_mfma_block expects, and how many of its
 // workgroups a compute unit holds at a time.
 extern "C" int qvl_attn_mfma_block_tiles() { return BLK_WAVES * BLK_CT; }

@@ -123,7 +123,9 @@ def try_attention(q, k_cache, v_cache, block_table, step, num_q_heads: int, wind
     else:
         scratch = None
         if nsplit > 1:
-            scratch = torch.empty(num_tiles * nkv * nsplit * 16 * (hd + 4), dtype=torch.float32, device=q.device)
+            floats = _fn("attention_mfma", "qvl_attn_mfma_scratch_floats", [_c_int] * 3, defines)
+            floats.restype = ctypes.c_longlong
+            scratch = torch.empty(int(floats(num_tiles, nkv, nsplit)), dtype=torch.float32, device=q.device)
         fn = _fn("attention_mfma", "qvl_attn_mfma_coop",
                  [_c_ptr] * 4 + [_c_int] + [_c_ptr] * 4 + [_c_int, _c_ptr, _c_ptr] + [_c_int] * 4
                  + [_c_float, _c_int, _c_int, _c_ptr], defines)

@@ -14,12 +14,12 @@ import torch
 
 from .kernels import _check, _fn, _ptr, _stream, dtype_code
 
-__all__ = ["resident_product", "takes_resident", "qkv_rope_product", "takes_qkv_rope", "try_streaming", "RESIDENT_ROWS", "RESIDENT_NORM_K", "MAX_ROWS",
+__all__ = ["resident_product", "takes_resident", "qkv_rope_product", "takes_qkv_rope", "try_streaming", "RESIDENT_ROWS", "resident_norm_k", "MAX_ROWS",
            "STORE", "RESIDUAL", "SWIGLU"]
 
 MAX_ROWS = 32            # the streaming kernel's limit in use
 RESIDENT_ROWS = 16       # up to here the resident kernel runs
-RESIDENT_NORM_K = 4096   # the folded norm needs the whole row in one pass of the block
+_pass_k = None
 STORE, RESIDUAL, SWIGLU = 0, 1, 2
 _c_int, _c_float, _c_ptr = ctypes.c_int, ctypes.c_float, ctypes.c_void_p
 _cu_count = {}
@@ -36,11 +36,20 @@ def _rows_aligned(t: torch.Tensor, elems: int) -> bool:
     return t.stride(1) == 1 and t.stride(0) % elems == 0 and t.data_ptr() % 16 == 0
 
 
+def resident_norm_k() -> int:
+    """The longest row whose norm the resident kernel folds in: the whole row must fit one pass of
+    the block (the kernel's own constant)."""
+    global _pass_k
+    if _pass_k is None:
+        _pass_k = int(_fn("gemm_resident", "qvl_gemm_resident_pass_k", [])())
+    return _pass_k
+
+
 def takes_resident(m: int, k: int, weight: torch.Tensor, *, norm: bool = False) -> bool:
     """Whether the resident kernel takes a product of ``m`` rows with this weight."""
     if m > RESIDENT_ROWS or k % 8 or weight.dtype != torch.bfloat16 or not _rows_aligned(weight, 8):
         return False
-    return not norm or k <= RESIDENT_NORM_K
+    return not norm or k <= resident_norm_k()
 
 
 def resident_product(weight: torch.Tensor, *, x: Optional[torch.Tensor] = None, h: Optional[torch.Tensor] = None,
