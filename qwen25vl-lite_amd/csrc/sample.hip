@@ -54,10 +54,49 @@ __device__ uint32_t threshold_search(const float* sc, int V, float mx, float tar
   return t;
 }
 
+// A row's largest logit, found by ARGMAX_SPLITS blocks side by side (one block for a row of a
+// hundred and fifty thousand logits is slower than the step's other kernels together): block s
+// scans the logits s * per .. (s + 1) * per - 1 and leaves (value, index), the lowest index among
+// equals; the row's block below picks among the splits, again the lowest index among equals.
+#define ARGMAX_SPLITS 32
+struct ArgmaxPart {
+  float value;
+  int index;
+};
+
+__global__ __launch_bounds__(256) void argmax_parts_kernel(const float* __restrict__ logits,
+                                                            ArgmaxPart* __restrict__ parts, int V) {
+  __shared__ float vals[4];
+  __shared__ int idxs[4];
+  const int m = blockIdx.y, s = blockIdx.x;
+  const int per = (V + ARGMAX_SPLITS - 1) / ARGMAX_SPLITS;
+  const int lo = s * per, hi = min(V, lo + per);
+  const float* lg = logits + (size_t)m * V;
+  float bv = -INFINITY;
+  int bi = V;
+  for (int i = lo + threadIdx.x; i < hi; i += blockDim.x) {
+    const float x = lg[i];
+    if (x > bv) { bv = x; bi = i; }   // indices rise within a thread: the first of equals stays
+  }
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(bv, o, QVL_WAVE);
+    const int oi = __shfl_xor(bi, o, QVL_WAVE);
+    if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+  }
+  if ((threadIdx.x & 63) == 0) { vals[threadIdx.x >> 6] = bv; idxs[threadIdx.x >> 6] = bi; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 4; ++w)
+      if (vals[w] > bv || (vals[w] == bv && idxs[w] < bi)) { bv = vals[w]; bi = idxs[w]; }
+    parts[(size_t)m * ARGMAX_SPLITS + s] = ArgmaxPart{bv, bi};
+  }
+}
+
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float* __restrict__ logits,
                                                                      float* __restrict__ scores,
                                                                      const RowParams* __restrict__ params,
                                                                      const int* __restrict__ prev_ids,
+                                                                     const ArgmaxPart* __restrict__ parts,
                                                                      int* __restrict__ out, int V) {
   __shared__ float red[17];
   __shared__ float sums[SAMPLE_THREADS];
@@ -100,6 +139,21 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float
     __syncthreads();
   }
 
+  if (greedy && !penal && parts) {
+    // the splits have scanned the row already
+    if (tid < 64) {
+      float bv = -INFINITY;
+      int bi = V;
+      if (tid < ARGMAX_SPLITS) { bv = parts[(size_t)m * ARGMAX_SPLITS + tid].value; bi = parts[(size_t)m * ARGMAX_SPLITS + tid].index; }
+      for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(bv, o, QVL_WAVE);
+        const int oi = __shfl_xor(bi, o, QVL_WAVE);
+        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+      }
+      if (tid == 0) out[m] = bi < V ? bi : 0;
+    }
+    return;
+  }
   if (greedy) {
     // argmax, the lowest index among equals
     float bv = -INFINITY;
@@ -193,13 +247,24 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float
   }
 }
 
-extern "C" int qvl_sample_rows(const void* logits, void* scores, const void* params, const void* prev_ids, void* out,
-                               int M, int V, hipStream_t stream) {
+// parts: null, or room for M * qvl_sample_argmax_part_bytes() bytes: then the rows' largest logits
+// are found by several blocks each first (worth it when some row is greedy without penalties).
+extern "C" int qvl_sample_rows(const void* logits, void* scores, const void* params, const void* prev_ids,
+                               void* parts, void* out, int M, int V, hipStream_t stream) {
   if (M <= 0) return QVL_OK;
   if (V <= 0) return QVL_ERR_SHAPE;
+  if (M > 65535) return QVL_ERR_LIMIT;
+  if (parts) {
+    hipLaunchKernelGGL(argmax_parts_kernel, dim3(ARGMAX_SPLITS, M), dim3(256), 0, stream, (const float*)logits,
+                       (ArgmaxPart*)parts, V);
+    if (hipGetLastError() != hipSuccess) return QVL_ERR_LAUNCH;
+  }
   hipLaunchKernelGGL(sample_rows_kernel, dim3(M), dim3(SAMPLE_THREADS), 0, stream, (const float*)logits,
-                     (float*)scores, (const RowParams*)params, (const int*)prev_ids, (int*)out, V);
+                     (float*)scores, (const RowParams*)params, (const int*)prev_ids, (const ArgmaxPart*)parts,
+                     (int*)out, V);
   return qvl_launch_status();
 }
+
+extern "C" int qvl_sample_argmax_part_bytes() { return (int)(ARGMAX_SPLITS * sizeof(ArgmaxPart)); }
 
 extern "C" int qvl_sample_params_size() { return (int)sizeof(RowParams); }

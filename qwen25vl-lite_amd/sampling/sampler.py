@@ -62,8 +62,8 @@ def sample_rows(logits: torch.Tensor, params: Sequence[SamplingParams], prev_ids
         rows[i] = (p.temperature, p.top_p, p.min_p, u, p.repetition_penalty, p.presence_penalty,
                    p.frequency_penalty, p.top_k if p.top_k else -1, begin, len(flat))
     fn = _fn("sample", "qvl_sample_rows",
-             [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
-              ctypes.c_int, ctypes.c_void_p])
+             [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+              ctypes.c_int, ctypes.c_int, ctypes.c_void_p])
     dev = logits.device
     with torch.cuda.device(dev):
         packed = np.concatenate([rows.view(np.int32), np.asarray(flat or [0], np.int32)])
@@ -72,6 +72,13 @@ def sample_rows(logits: torch.Tensor, params: Sequence[SamplingParams], prev_ids
         need_scores = any(p.temperature > 0 or len(flat) for p in params)
         scores = torch.empty_like(logits) if need_scores else logits
         out = torch.empty(m, dtype=torch.int32, device=dev)
+        # a greedy row without penalties is a plain argmax: several blocks scan it side by side
+        parts = None
+        if any(p.temperature <= 0 and p.repetition_penalty == 1.0 and p.presence_penalty == 0.0
+               and p.frequency_penalty == 0.0 for p in params):
+            part_bytes = int(_fn("sample", "qvl_sample_argmax_part_bytes", [])())
+            parts = torch.empty(m * part_bytes, dtype=torch.uint8, device=dev)
         _check(fn(logits.data_ptr(), scores.data_ptr(), buf.data_ptr(), buf[n_row_words:].data_ptr(),
-                  out.data_ptr(), m, vocab, _stream()), "sample_rows")
+                  parts.data_ptr() if parts is not None else None, out.data_ptr(), m, vocab, _stream()),
+               "sample_rows")
         return out.cpu().tolist()

@@ -174,6 +174,18 @@ def test_sampler_kernel_against_plain():
                 cdf = torch.cumsum(probs, 0) / probs.sum()
                 assert probs[got[i]] > 0 and min(abs(cdf[got[i]] - us[i]), abs(cdf[got[i]] - probs[got[i]] - us[i])) < 1e-5, \
                     (trial, i, got[i], want)
+    # greedy rows: the lowest index among equal maxima, wherever in the row they lie (the row is
+    # scanned in pieces), for a vocabulary that is no multiple of anything
+    vocab = 152064 + 7
+    rows = torch.randn(4, vocab, generator=g)
+    top = rows.max() + 1
+    spots = [[5, 70000, 152070], [152070], [4752, 4753, 9504], [0, 152070]]
+    for r, where in enumerate(spots):
+        rows[r, where] = top
+    greedy = [SamplingParams(temperature=0.0)] * 3 + [SamplingParams(temperature=0.0, presence_penalty=0.5)]
+    got = sample_rows(rows.cuda(), greedy, [[], [], [], [0]], [0, 0, 0, 1])
+    assert got == [5, 152070, 4752, 152070]        # the last row's token 0 is pushed down by its penalty
+
     # the distribution itself: many draws of one row follow the filtered probabilities
     p = SamplingParams(temperature=1.0, top_k=4)
     row = torch.tensor([2.0, 1.0, 0.5, 0.0, -1.0, -3.0])
