@@ -37,7 +37,7 @@ SIZES = {   # layer sizes of BASELINE.json's configs[3], [2] and [4]
 }
 
 
-def seven_b_config(layers=None, size="7b"):
+def decoder_config(layers=None, size="7b"):
     """configs[2] of BASELINE.json (or another of its sizes) as a config.json dictionary."""
     raw = {
         "architectures": ["Qwen2_5_VLForConditionalGeneration"], "model_type": "qwen2_5_vl",
@@ -99,7 +99,7 @@ def main(argv=None) -> int:
     from qwen25vl_lite_amd.config import dtype_from_name
     from qwen25vl_lite_amd.weights import fill_random
 
-    cfg = Qwen25VLConfig.from_dict(seven_b_config(args.layers, args.size))
+    cfg = Qwen25VLConfig.from_dict(decoder_config(args.layers, args.size))
     t = cfg.text_config
     dtype = dtype_from_name(args.dtype)
     model = build_model(cfg, dtype, "cuda:0")
