@@ -151,11 +151,14 @@ class RadixPrefixCache:
             self._drop(leaves[0])
 
     def evict(self, pages_wanted: int) -> int:
-        """Evict unused leaves, oldest first, until every pool has ``pages_wanted`` free pages
-        or nothing evictable is left.  Returns the number of nodes evicted."""
+        """Evict unused leaves, oldest first, until every pool has ``pages_wanted`` free pages or
+        no leaf is left whose eviction would free a page.  A leaf whose pages a running request
+        still holds (the one that registered it) stays: dropping it would give nothing back and
+        only lose the entry.  Returns the number of nodes evicted."""
         evicted = 0
         while any(pool.num_free < pages_wanted for pool in self.pools):
-            leaves = self._evictable_leaves()
+            leaves = [nid for nid in self._evictable_leaves()
+                      if any(pool.refcount(self.nodes[nid].pages[g]) == 1 for g, pool in enumerate(self.pools))]
             if not leaves:
                 break
             evicted += self._drop(leaves[0])

@@ -165,6 +165,29 @@ def test_pressure_evicts_unused_prefixes_but_not_used_ones():
     assert cm.pages_in_use() == [0]
 
 
+def test_pressure_keeps_entries_whose_pages_would_not_come_back():
+    """A running request's registered prefix has no user, but evicting it frees nothing (the
+    request still holds the pages): under pressure it stays, so that a later request can find it."""
+    cm = _manager(windows=(None,), pages=5, page_size=4, seqs=3)
+    toks = list(range(200, 212))
+    cm.admit("a")
+    cm.reserve("a", 12)
+    cm.commit("a", 12)
+    assert cm.register_prefix("a", toks) == 3        # a keeps running and holding its three pages
+    cm.admit("b")
+    with pytest.raises(OutOfPages):
+        cm.reserve("b", 12)                           # 2 free pages, 3 wanted: nothing to gain by evicting
+    assert len(cm.prefix_cache) == 3, "the entries are still there"
+    cm.release("b")
+    cm.admit("c")
+    assert cm.adopt_prefix("c", toks + [7]) == 12     # and are found
+    cm.release("a")
+    cm.release("c")
+    cm.check()
+    cm.prefix_cache.evict(5)                          # now the cache alone holds them: they come back
+    assert cm.pages_in_use() == [0] and len(cm.prefix_cache) == 0
+
+
 def test_slots():
     cm = _manager(seqs=2)
     s0, s1 = cm.admit("a"), cm.admit("b")

@@ -105,6 +105,43 @@ def test_decode_graphs_with_padding_rows(model_dirs, name, dtype):
     assert llm.runner.cache.pages_in_use() == [0] * len(llm.runner.cache.groups)
 
 
+@pytest.mark.parametrize("name, seed", [("A_sharp", 0), ("A_sharp", 1), ("C_sharp", 2)])
+def test_everything_at_once(model_dirs, name, seed):
+    """A server's day in small: requests of random lengths, some sharing a prefix, more of them than
+    request slots, so few pages that some are preempted and computed again, decode steps from HIP
+    graphs with padding rows, the prefix cache on (model A) or a windowed group giving pages back
+    (model C).  In float32 every request's tokens are the plain implementation's, and all pages
+    come back."""
+    import random
+    from qwen25vl_lite_amd import LLM, SamplingParams
+
+    d = model_dirs[name]
+    vocab = {"A": 256, "C": 300}[name[0]]
+    rng = random.Random(seed)
+    shared = random_tokens(40, vocab, 500 + seed)
+    prompts, params = [], []
+    for i in range(9):
+        n = 8 if i == 0 else rng.randint(2, 60)
+        body = random_tokens(n, vocab, 600 + 10 * seed + i)
+        # the first request holds the shared prefix for as long as it runs; two later ones find it
+        prompts.append(shared + body if i in (0, 6, 7) else body)
+        params.append(SamplingParams(temperature=0.0, max_tokens=45 if i == 0 else rng.randint(3, 40),
+                                     ignore_eos=True))
+    llm = LLM(d, dtype="float32", num_blocks=18, block_size=16, max_num_seqs=5, max_num_batched_tokens=48,
+              hip_graph=True, enable_prefix_cache=True)
+    outs = llm.generate(prompts, params)
+    stats = llm.engine.stats()
+    assert stats["preemptions"] > 0, stats
+    assert len(llm.runner.graphs.graphs) >= 2
+    if name[0] == "A":
+        assert stats["prefix_cache_hits"] > 0, stats
+    for prompt, p, out in zip(prompts, params, outs):
+        assert out.output_token_ids == _plain_greedy(d, prompt, p.max_tokens), (len(prompt), p.max_tokens)
+    llm.runner.cache.check()
+    cached = len(llm.runner.cache.prefix_cache) if llm.runner.cache.prefix_cache else 0
+    assert llm.runner.cache.pages_in_use()[0] == cached
+
+
 def test_prefix_reuse_gives_the_same_tokens(model_dirs):
     # reference tests/test_chunked_prefill.py:193-227, tests/test_engine.py:57-106
     from qwen25vl_lite_amd import LLM, SamplingParams
