@@ -50,7 +50,7 @@ def cmd_generate(args) -> int:
         # reference cli.py:271-274
         print("--prompt-token-ids is required (this CLI does not bundle a tokenizer)", file=sys.stderr)
         return 2
-    prompts = [[int(t) for t in part.split(",") if t.strip()] for part in args.prompt_token_ids.split(";")]
+    prompts = _read_prompts(args.prompt_token_ids)
     llm = _llm(args)
     params = SamplingParams(temperature=args.temperature, top_p=args.top_p, top_k=args.top_k,
                             max_tokens=args.max_tokens, seed=args.seed, ignore_eos=args.ignore_eos)
@@ -58,6 +58,21 @@ def cmd_generate(args) -> int:
     for out in outs:
         print(out.output_token_ids)
     return 0
+
+
+def _read_prompts(arg: str):
+    """``"1,2,3"``, several prompts separated by ``;``, or the path of a JSON file that holds a
+    list of token ids or a list of such lists."""
+    import json
+    import os
+
+    if os.path.isfile(arg):
+        with open(arg) as f:
+            data = json.load(f)
+        if data and not isinstance(data[0], list):
+            data = [data]
+        return [[int(t) for t in prompt] for prompt in data]
+    return [[int(t) for t in part.split(",") if t.strip()] for part in arg.split(";")]
 
 
 def cmd_bench(args) -> int:
@@ -126,7 +141,7 @@ def build_parser() -> argparse.ArgumentParser:
     p = sub.add_parser("generate", help="one-shot generation from token ids")
     add_model_opts(p)
     add_engine_opts(p)
-    p.add_argument("--prompt-token-ids", default=None, help='"1,2,3"; several prompts separated by ";"')
+    p.add_argument("--prompt-token-ids", default=None, help='"1,2,3"; several prompts separated by ";"; or a JSON file with a list of lists')
     p.add_argument("--temperature", type=float, default=0.0)
     p.add_argument("--top-p", type=float, default=1.0)
     p.add_argument("--top-k", type=int, default=-1)
