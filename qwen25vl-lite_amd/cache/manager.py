@@ -157,6 +157,39 @@ class CacheManager:
             out.append(page * ps + p % ps)
         return out
 
+    # ------------------------------------------------------------------ forking
+    def fork(self, src_id, dst_id) -> List[Tuple[int, int, int]]:
+        """A new request ``dst_id`` that continues from where ``src_id`` stands (several
+        continuations of one prompt).  Pages that are full are shared (one more holder each); the
+        page still being filled gets a copy of its own, because both requests will write to it.
+        Returns the copies the caller has to make on the device, as ``(group, from page, to page)``.
+        Raises :class:`OutOfPages` / :class:`OutOfSlots` and changes nothing if there is no room."""
+        src = self.requests[src_id]
+        full = src.num_tokens // self.page_size
+        partial = src.num_tokens % self.page_size != 0
+        if partial:
+            if self.prefix_cache is not None and any(pool.num_free < 1 for pool in self.pools):
+                self.prefix_cache.evict(1)
+            for pool in self.pools:
+                if pool.num_free < 1:
+                    raise OutOfPages("no page free for the copy of the page being filled")
+        self.admit(dst_id)
+        dst = self.requests[dst_id]
+        copies: List[Tuple[int, int, int]] = []
+        for g, table in enumerate(src.tables):
+            shared = list(table[:full])
+            self.pools[g].fork([p for p in shared if p >= 0])
+            if partial:
+                fresh = self.pools[g].allocate(1)[0]
+                copies.append((g, table[full], fresh))
+                shared.append(fresh)
+            dst.tables[g] = shared
+        dst.num_tokens = src.num_tokens
+        if src.prefix_nodes and self.prefix_cache is not None:
+            self.prefix_cache.add_users(src.prefix_nodes)
+            dst.prefix_nodes = list(src.prefix_nodes)
+        return copies
+
     # ------------------------------------------------------------------ shared prefixes
     def adopt_prefix(self, req_id, tokens: Sequence[int], extra_keys: Optional[Sequence] = None) -> int:
         """Reuse cached pages for the longest known prefix, keeping at least one token to

@@ -84,6 +84,11 @@ class RadixPrefixCache:
         pages = [[self.nodes[nid].pages[g] for nid in path] for g in range(len(self.pools))]
         return len(path) * self.page_size, path, pages
 
+    def add_users(self, node_ids: Sequence[int]) -> None:
+        """One more request uses these nodes (a fork of a request that adopted them)."""
+        for nid in node_ids:
+            self.nodes[nid].users += 1
+
     def release(self, node_ids: Sequence[int]) -> None:
         """A request that adopted these nodes is done with them."""
         for nid in node_ids:

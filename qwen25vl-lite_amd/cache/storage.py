@@ -30,5 +30,12 @@ class KVStorage:
             self.k.append(torch.zeros((g.num_layers, num_pages, nkv, page_size, hd), dtype=dtype, device=device))
             self.v.append(torch.zeros((g.num_layers, num_pages, nkv, hd, page_size), dtype=dtype, device=device))
 
+    def copy_pages(self, group: int, src: Sequence[int], dst: Sequence[int]) -> None:
+        """Keys and values of pages ``src`` into pages ``dst`` of a group, in all of its layers
+        (reference cache.py:537-545)."""
+        from ..ops import kernels
+        kernels.copy_pages(self.k[group], src, dst)
+        kernels.copy_pages(self.v[group], src, dst)
+
     def nbytes(self) -> int:
         return sum(t.numel() * t.element_size() for t in self.k + self.v)

@@ -314,3 +314,26 @@ extern "C" int qvl_swiglu(const void* x, void* out, int N, int I, int dtype, int
     return QVL_ERR_DTYPE;
   return qvl_launch_status();
 }
+
+// ---------------------------------------------------------------------------------------
+// Page copy (reference cache.py:537-545): page src[i] -> page dst[i] in every layer of a cache
+// tensor [layers, pages, page_bytes].  Used when a request is forked: whole pages are shared,
+// the page being filled is copied.
+// ---------------------------------------------------------------------------------------
+__global__ void copy_pages_kernel(char* __restrict__ cache, size_t layer_bytes, int page_bytes,
+                                  const int* __restrict__ src, const int* __restrict__ dst) {
+  const int i = blockIdx.x, layer = blockIdx.y;
+  const uint4* from = reinterpret_cast<const uint4*>(cache + layer * layer_bytes + (size_t)src[i] * page_bytes);
+  uint4* to = reinterpret_cast<uint4*>(cache + layer * layer_bytes + (size_t)dst[i] * page_bytes);
+  for (int c = threadIdx.x; c < page_bytes / 16; c += blockDim.x) to[c] = from[c];
+}
+
+extern "C" int qvl_copy_pages(void* cache, long long layer_bytes, int page_bytes, const void* src, const void* dst,
+                              int n, int layers, hipStream_t stream) {
+  if (n <= 0 || layers <= 0) return QVL_OK;
+  if (page_bytes <= 0 || page_bytes % 16 || layer_bytes < page_bytes || ((uintptr_t)cache & 15)) return QVL_ERR_SHAPE;
+  if (layers > 65535) return QVL_ERR_LIMIT;
+  hipLaunchKernelGGL(copy_pages_kernel, dim3(n, layers), dim3(256), 0, stream, (char*)cache, (size_t)layer_bytes,
+                     page_bytes, (const int*)src, (const int*)dst);
+  return qvl_launch_status();
+}

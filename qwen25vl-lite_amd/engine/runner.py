@@ -67,6 +67,17 @@ class ModelRunner:
     def release(self, req_id) -> None:
         self.cache.release(req_id)
 
+    def fork(self, src_id, dst_id) -> None:
+        """``dst_id`` continues from where ``src_id`` stands: full pages shared, the page being
+        filled copied, per-request state rows copied."""
+        for group, src_page, dst_page in self.cache.fork(src_id, dst_id):
+            self.storage.copy_pages(group, [src_page], [dst_page])
+        a, b = self.cache.slot_of(src_id), self.cache.slot_of(dst_id)
+        for state in self.states:
+            if state is not None:
+                state[b].copy_(state[a])
+        self.cache.take_fresh(dst_id)      # the copied state must not be cleared
+
     def _clear_state(self, entries: Sequence[StepEntry]) -> None:
         for e in entries:
             if self.cache.take_fresh(e.req_id):

@@ -8,13 +8,13 @@ There is no CPU path and no library stand-in: a tensor that is not on the GPU is
 from __future__ import annotations
 
 import ctypes
-from typing import Dict, Optional, Tuple
+from typing import Dict, Optional, Sequence, Tuple
 
 import torch
 
 from .library import load_library
 
-__all__ = ["rope_table", 
+__all__ = ["rope_table", "copy_pages", 
     "KernelError", "embed_gather", "add_rmsnorm", "rope_kv_write", "paged_attention_generic", "swiglu",
     "gemm_f32", "dtype_code",
 ]
@@ -192,6 +192,25 @@ def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, freq_row: torch.
     _check(fn(_ptr(positions), positions.stride(0), _ptr(inv_freq), _ptr(freq_row), _ptr(out), int(n), rot_half,
               _stream()), "rope_table")
     return out
+
+
+def copy_pages(cache: torch.Tensor, src: Sequence[int], dst: Sequence[int]) -> None:
+    """Copy page ``src[i]`` to page ``dst[i]`` in every layer of ``cache [layers, pages, ...]``
+    (the pages must not overlap between the two lists)."""
+    _dev(cache)
+    _need(cache.dim() >= 3 and cache.is_contiguous(), "cache must be contiguous [layers, pages, ...]")
+    _need(len(src) == len(dst), "as many source as destination pages are needed")
+    if not src:
+        return
+    pages = cache.shape[1]
+    _need(all(0 <= int(p) < pages for p in list(src) + list(dst)), "a page id is outside the cache")
+    _need(not set(map(int, src)) & set(map(int, dst)), "a page is both copied from and copied to")
+    page_bytes = cache[0, 0].numel() * cache.element_size()
+    idx = torch.tensor([list(map(int, src)), list(map(int, dst))], dtype=torch.int32, device=cache.device)
+    fn = _fn("elementwise", "qvl_copy_pages",
+             [_c_ptr, ctypes.c_longlong, _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(cache), pages * page_bytes, page_bytes, _ptr(idx[0]), _ptr(idx[1]), len(src), cache.shape[0],
+              _stream()), "copy_pages")
 
 
 def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,

@@ -188,6 +188,45 @@ def test_pressure_keeps_entries_whose_pages_would_not_come_back():
     assert cm.pages_in_use() == [0] and len(cm.prefix_cache) == 0
 
 
+def test_fork_shares_full_pages_and_copies_the_one_being_filled():
+    cm = _manager(windows=(None, 6), pages=8, page_size=4, seqs=3)
+    cm.admit("a")
+    cm.reserve("a", 10)
+    cm.commit("a", 10)                                  # pages 0..1 full, page 2 half full; window 6 gave page 0 back
+    assert cm.table("a", 1)[0] == -1
+    copies = cm.fork("a", "b")
+    assert [(g, src) for g, src, _ in copies] == [(0, cm.table("a", 0)[2]), (1, cm.table("a", 1)[2])]
+    for g, src, dst in copies:
+        assert dst != src and cm.table("b", g)[2] == dst
+    assert cm.table("b", 0)[:2] == cm.table("a", 0)[:2] and cm.table("b", 1)[:2] == cm.table("a", 1)[:2]
+    assert cm.num_tokens("b") == 10 and cm.slot_of("b") != cm.slot_of("a")
+    cm.check()
+    for req in ("a", "b"):                               # both go on, each into its own pages
+        cm.reserve(req, 14)
+        cm.commit(req, 14)
+    assert cm.table("a", 0)[3] != cm.table("b", 0)[3]
+    cm.check()
+    cm.release("a")
+    cm.check()
+    cm.release("b")
+    assert cm.pages_in_use() == [0, 0]
+    # no room for the copy: nothing changes
+    cm.admit("c")
+    cm.reserve("c", 30)
+    cm.commit("c", 30)
+    with pytest.raises(OutOfPages):
+        cm.fork("c", "d")
+    assert "d" not in cm.requests
+    cm.check()
+    # at a page boundary nothing is copied
+    cm.release("c")
+    cm.admit("e")
+    cm.reserve("e", 8)
+    cm.commit("e", 8)
+    assert cm.fork("e", "f") == []
+    cm.check()
+
+
 def test_slots():
     cm = _manager(seqs=2)
     s0, s1 = cm.admit("a"), cm.admit("b")

@@ -142,6 +142,36 @@ def test_everything_at_once(model_dirs, name, seed):
     assert llm.runner.cache.pages_in_use()[0] == cached
 
 
+@pytest.mark.parametrize("name", ["B_sharp", "C_sharp"])
+def test_forked_request_continues_on_its_own_pages(model_dirs, name):
+    """A request forked in the middle of a page (reference cache.py:537-545 copies blocks for
+    this): the two continuations share the full pages, each writes to its own copy of the page
+    being filled, and each one's logits are those of its own whole sequence."""
+    from qwen25vl_lite_amd import LLM
+    from qwen25vl_lite_amd.engine.batch import StepEntry
+
+    d = model_dirs[name]
+    vocab = {"B": 509, "C": 300}[name[0]]
+    runner = LLM(d, dtype="float32", num_blocks=12, block_size=16, max_num_seqs=3, enable_prefix_cache=False).runner
+    prompt = random_tokens(53, vocab, 31)
+    tails = {"a": random_tokens(20, vocab, 32), "b": random_tokens(20, vocab, 33)}
+    runner.admit("a")
+    runner.execute([StepEntry("a", prompt, 0, [])])
+    runner.fork("a", "b")
+    got = {"a": [], "b": []}
+    for i in range(20):
+        logits = runner.execute([StepEntry(r, [tails[r][i]], 53 + i, [0]) for r in ("b", "a")])
+        got["b"].append(logits[0].cpu())
+        got["a"].append(logits[1].cpu())
+    for r in ("a", "b"):
+        want = plain_model_logits(d, prompt + tails[r])[53:]
+        assert torch.allclose(torch.stack(got[r]), want, atol=1e-4, rtol=1e-3), r
+    runner.cache.check()
+    runner.release("a")
+    runner.release("b")
+    assert runner.cache.pages_in_use() == [0] * len(runner.cache.groups)
+
+
 def test_prefix_reuse_gives_the_same_tokens(model_dirs):
     # reference tests/test_chunked_prefill.py:193-227, tests/test_engine.py:57-106
     from qwen25vl_lite_amd import LLM, SamplingParams
