@@ -159,8 +159,9 @@ template <typename TI, typename T>
 __global__ void rope_kv_write_kernel(const TI* __restrict__ x, int x_stride, const float* __restrict__ bias,
                                      const int* __restrict__ pos, int pos_stride,
                                      const float* __restrict__ inv_freq, const int* __restrict__ freq_row,
-                                     const int* __restrict__ slot, T* __restrict__ q_out, T* __restrict__ kc,
-                                     T* __restrict__ vc, int nq, int nkv, int hd, int rot_half, int ps) {
+                                     const float2* __restrict__ cs, const int* __restrict__ slot,
+                                     T* __restrict__ q_out, T* __restrict__ kc, T* __restrict__ vc, int nq, int nkv,
+                                     int hd, int rot_half, int ps) {
   const int n = blockIdx.x;
   const int hh = blockIdx.y;
   const TI* src = x + (size_t)n * x_stride + (size_t)hh * hd;
@@ -190,11 +191,17 @@ __global__ void rope_kv_write_kernel(const TI* __restrict__ x, int x_stride, con
   for (int f = threadIdx.x; f < rot_half; f += blockDim.x) {
     float x1 = ldf<TI>(src + f) + (b ? b[f] : 0.f);
     float x2 = ldf<TI>(src + f + rot_half) + (b ? b[f + rot_half] : 0.f);
-    const int row = freq_row[f];
     float c = 1.f, s = 0.f;
-    if (row >= 0) {
-      const float ang = (float)pos[(size_t)row * pos_stride + n] * inv_freq[f];
-      sincosf(ang, &s, &c);
+    if (cs) {  // the step's table of cosines and sines: every head and layer reads the same values
+      const float2 v = cs[(size_t)n * rot_half + f];
+      c = v.x;
+      s = v.y;
+    } else {
+      const int row = freq_row[f];
+      if (row >= 0) {
+        const float ang = (float)pos[(size_t)row * pos_stride + n] * inv_freq[f];
+        sincosf(ang, &s, &c);
+      }
     }
     stf<T>(dst + f, x1 * c - x2 * s);
     stf<T>(dst + f + rot_half, x2 * c + x1 * s);
@@ -203,8 +210,10 @@ __global__ void rope_kv_write_kernel(const TI* __restrict__ x, int x_stride, con
     stf<T>(dst + d, ldf<TI>(src + d) + (b ? b[d] : 0.f));
 }
 
+// cs: null, or float32 [N, rot_half, 2] from qvl_rope_table (then pos, inv_freq and freq_row are not read).
 extern "C" int qvl_rope_kv_write(const void* x, int x_stride, const void* bias, const void* pos, int pos_stride,
-                                 const void* inv_freq, const void* freq_row, const void* slot, void* q_out, void* kc,
+                                 const void* inv_freq, const void* freq_row, const void* cs, const void* slot,
+                                 void* q_out, void* kc,
                                  void* vc, int N, int nq, int nkv, int hd, int rot_half, int ps, int in_dtype,
                                  int dtype, hipStream_t stream) {
   if (N <= 0) return QVL_OK;
@@ -217,8 +226,8 @@ extern "C" int qvl_rope_kv_write(const void* x, int x_stride, const void* bias, 
   if (in_dtype == ID && dtype == OD) {                                                                             \
     hipLaunchKernelGGL((rope_kv_write_kernel<TI, T>), grid, dim3(64), 0, stream, (const TI*)x, x_stride,           \
                        (const float*)bias, (const int*)pos, pos_stride, (const float*)inv_freq,                    \
-                       (const int*)freq_row, (const int*)slot, (T*)q_out, (T*)kc, (T*)vc, nq, nkv, hd, rot_half,   \
-                       ps);                                                                                        \
+                       (const int*)freq_row, (const float2*)cs, (const int*)slot, (T*)q_out, (T*)kc, (T*)vc, nq,   \
+                       nkv, hd, rot_half, ps);                                                                     \
     return qvl_launch_status();                                                                                    \
   }
   QVL_ROPE_CASE(0, 0, float, float)

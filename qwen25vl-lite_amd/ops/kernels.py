@@ -129,7 +129,7 @@ def rope_kv_write(x: torch.Tensor, bias: Optional[torch.Tensor], positions: torc
                   freq_row: torch.Tensor, slots: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
                   v_cache: Optional[torch.Tensor], num_q_heads: int, num_kv_heads: int, head_dim: int,
                   page_size: int, out_dtype: Optional[torch.dtype] = None,
-                  q_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                  q_out: Optional[torch.Tensor] = None, cs: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Rotate queries and keys, write keys and values into their page slots, return queries.
 
     ``x`` may be float32 while queries and the cache are bfloat16 (``out_dtype``): the bias is
@@ -139,6 +139,8 @@ def rope_kv_write(x: torch.Tensor, bias: Optional[torch.Tensor], positions: torc
     int32 ``[rows, N]``; ``freq_row[f]`` names the row that frequency ``f`` uses (-1: none).
     ``k_cache`` is one layer's ``[pages, nkv, page_size, hd]``, ``v_cache`` its
     ``[pages, nkv, hd, page_size]``.  With ``num_kv_heads == 0`` only queries are rotated.
+    ``cs`` is :func:`rope_table` of the same positions and tables, if the caller has it: the
+    kernel then reads the cosines and sines instead of computing them for every head.
     """
     _dev(x, bias, positions, inv_freq, freq_row, slots, k_cache, v_cache, q_out)
     n = x.shape[0]
@@ -168,11 +170,15 @@ def rope_kv_write(x: torch.Tensor, bias: Optional[torch.Tensor], positions: torc
     if q_out is None:
         q_out = torch.empty((n, nq * hd), dtype=odt, device=x.device)
     _need(q_out.shape == (n, nq * hd) and q_out.dtype == odt and q_out.is_contiguous(), "q_out must be [N, nq hd]")
+    if cs is not None:
+        _dev(cs)
+        _need(cs.dtype == torch.float32 and cs.is_contiguous() and cs.dim() == 3 and cs.shape[0] >= n
+              and tuple(cs.shape[1:]) == (rot_half, 2), "cs must be float32 [N, rot/2, 2]")
     fn = _fn("elementwise", "qvl_rope_kv_write",
-             [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+             [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
               _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
     _check(fn(_ptr(x), x.stride(0), _ptr(bias), _ptr(positions), positions.stride(0), _ptr(inv_freq),
-              _ptr(freq_row), _ptr(slots), _ptr(q_out), _ptr(k_cache), _ptr(v_cache), n, nq, nkv, hd, rot_half,
+              _ptr(freq_row), _ptr(cs), _ptr(slots), _ptr(q_out), _ptr(k_cache), _ptr(v_cache), n, nq, nkv, hd, rot_half,
               int(page_size), dtype_code(x.dtype), dtype_code(odt), _stream()), "rope_kv_write")
     return q_out
 

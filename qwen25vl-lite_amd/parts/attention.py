@@ -104,15 +104,24 @@ class PagedAttention(Mixer):
         # Projections are written out in float32 (the accumulator, unrounded): bias, rotation and
         # the residual sum then happen in float32 and each stored value is rounded once.
         qkv = linear(x, self.w_in, out_dtype=torch.float32)
+        cs = self._rotation_table(step, inv_freq, freq_row, qkv.shape[0])
         return kernels.rope_kv_write(
             qkv, self.b_in, step.positions, inv_freq, freq_row,
             group.slot_mapping if write else None, slot.k_cache if write else None, slot.v_cache if write else None,
-            self.nq, self.nkv if write else 0, self.hd, group.page_size, out_dtype=self.dtype)
+            self.nq, self.nkv if write else 0, self.hd, group.page_size, out_dtype=self.dtype, cs=cs)
+
+    def _rotation_table(self, step, inv_freq, freq_row, n: int) -> torch.Tensor:
+        """Cosines and sines of the step's angles: computed once per pass and position encoding,
+        by the first layer that needs them, and read by every head of every layer."""
+        key = ("rope_cs", self.position.table_key(self.hd))
+        cs = step.per_pass.get(key)
+        if cs is None:
+            cs = step.per_pass[key] = kernels.rope_table(step.positions, inv_freq, freq_row, n)
+        return cs
 
     def _project_few_rows(self, x, step, group, slot, write, inv_freq, freq_row) -> Optional[torch.Tensor]:
         """A decode step's few bfloat16 rows: projection, bias, rotation and cache write in one
-        kernel (the float32 sums never leave it).  The cosines and sines of the step's angles are
-        computed once per step and position encoding, by the first layer that needs them."""
+        kernel (the float32 sums never leave it)."""
         lazy = isinstance(x, NormedRows)
         m, k = x.shape
         if self.dtype != torch.bfloat16 or not skinny.takes_qkv_rope(
@@ -120,10 +129,7 @@ class PagedAttention(Mixer):
             return None
         if not lazy and (x.dtype != torch.bfloat16 or x.stride(1) != 1 or x.stride(0) % 8 or x.data_ptr() % 16):
             return None
-        key = ("rope_cs", self.position.table_key(self.hd))
-        cs = step.per_pass.get(key)
-        if cs is None:
-            cs = step.per_pass[key] = kernels.rope_table(step.positions, inv_freq, freq_row, m)
+        cs = self._rotation_table(step, inv_freq, freq_row, m)
         src = dict(h=x.h, norm_weight=x.weight, eps=x.eps) if lazy else dict(x=x)
         return skinny.qkv_rope_product(
             self.w_in, cs, bias=self.b_in, slots=group.slot_mapping if write else None,

@@ -79,6 +79,14 @@ def test_rope_kv_write(dtype, nq, nkv, hd, sections):
     untouched = torch.ones(pages * ps, dtype=torch.bool)
     untouched[slots.long()] = False
     assert kflat[untouched].abs().max() == 0 and vflat[untouched].abs().max() == 0
+    # with the step's table of cosines and sines in hand the kernel gives the very same values
+    cs = kernels.rope_table(pos.to(torch.int32).cuda(), inv.cuda(), rows.cuda(), n)
+    want_cs = torch.stack([torch.cos(pos[rows.long()].T.float() * inv), torch.sin(pos[rows.long()].T.float() * inv)], dim=-1)
+    assert torch.allclose(cs.cpu(), want_cs, atol=2e-4)
+    kc2, vc2 = torch.zeros_like(kc), torch.zeros_like(vc)
+    q2 = kernels.rope_kv_write(x.cuda(), bias.cuda(), pos.to(torch.int32).cuda(), inv.cuda(), rows.cuda(), slots.cuda(),
+                               kc2, vc2, nq, nkv, hd, ps, out_dtype=dtype, cs=cs)
+    assert torch.equal(q2, q) and torch.equal(kc2, kc) and torch.equal(vc2, vc)
     # position 0 leaves a head as it is; a negative slot writes nothing; rot < hd leaves the tail alone
     kc.zero_()
     q0 = kernels.rope_kv_write(x.cuda(), None, torch.zeros(3, n, dtype=torch.int32).cuda(), inv.cuda(), rows.cuda(),
