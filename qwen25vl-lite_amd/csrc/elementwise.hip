@@ -210,6 +210,79 @@ __global__ void rope_kv_write_kernel(const TI* __restrict__ x, int x_stride, con
     stf<T>(dst + d, ldf<TI>(src + d) + (b ? b[d] : 0.f));
 }
 
+// The same for float32 sums, bfloat16 outputs and the table of cosines and sines in hand, with
+// all widths multiples of 4 (the prompt portions of a bfloat16 run): a block per token, a thread
+// per 4 neighbouring channels, 16-byte loads and 8-byte stores.
+__global__ __launch_bounds__(256) void rope_kv_write_wide_kernel(
+    const float* __restrict__ x, int x_stride, const float* __restrict__ bias, const float2* __restrict__ cs,
+    const int* __restrict__ slot, bf16_t* __restrict__ q_out, bf16_t* __restrict__ kc, bf16_t* __restrict__ vc, int nq,
+    int nkv, int hd, int rot_half, int ps) {
+  const int n = blockIdx.x;
+  const float* src = x + (size_t)n * x_stride;
+  const int s = nkv ? slot[n] : -1;
+  const size_t page = s >= 0 ? (size_t)(s / ps) : 0, off = s >= 0 ? (size_t)(s % ps) : 0;
+  auto add_bias = [&](float4 v, int at) {
+    if (bias) {
+      const float4 b = *reinterpret_cast<const float4*>(bias + at);
+      v.x += b.x; v.y += b.y; v.z += b.z; v.w += b.w;
+    }
+    return v;
+  };
+  auto pack4 = [](float4 v) {
+    uint2 o;
+    o.x = (uint32_t)f32_to_bf16(v.x) | ((uint32_t)f32_to_bf16(v.y) << 16);
+    o.y = (uint32_t)f32_to_bf16(v.z) | ((uint32_t)f32_to_bf16(v.w) << 16);
+    return o;
+  };
+  // rotated heads: items (head, 4 frequencies)
+  const int per_head = rot_half / 4, rotated = (nq + nkv) * per_head;
+  for (int it = threadIdx.x; it < rotated; it += blockDim.x) {
+    const int hh = it / per_head, f = (it - hh * per_head) * 4;
+    bf16_t* dst;
+    if (hh < nq) {
+      dst = q_out + ((size_t)n * nq + hh) * hd;
+    } else {
+      if (s < 0) continue;
+      dst = kc + ((page * nkv + (hh - nq)) * ps + off) * hd;
+    }
+    const float4 x1 = add_bias(*reinterpret_cast<const float4*>(src + hh * hd + f), hh * hd + f);
+    const float4 x2 = add_bias(*reinterpret_cast<const float4*>(src + hh * hd + f + rot_half), hh * hd + f + rot_half);
+    const float4 c01 = *reinterpret_cast<const float4*>(cs + (size_t)n * rot_half + f);      // (c0, s0, c1, s1)
+    const float4 c23 = *reinterpret_cast<const float4*>(cs + (size_t)n * rot_half + f + 2);
+    const float4 lo = {x1.x * c01.x - x2.x * c01.y, x1.y * c01.z - x2.y * c01.w, x1.z * c23.x - x2.z * c23.y,
+                       x1.w * c23.z - x2.w * c23.w};
+    const float4 hi = {x2.x * c01.x + x1.x * c01.y, x2.y * c01.z + x1.y * c01.w, x2.z * c23.x + x1.z * c23.y,
+                       x2.w * c23.z + x1.w * c23.w};
+    *reinterpret_cast<uint2*>(dst + f) = pack4(lo);
+    *reinterpret_cast<uint2*>(dst + f + rot_half) = pack4(hi);
+  }
+  // channels past the rotation, unrotated
+  const int tail = (hd - 2 * rot_half) / 4;
+  for (int it = threadIdx.x; it < (nq + nkv) * tail; it += blockDim.x) {
+    const int hh = it / tail, d = 2 * rot_half + (it - hh * tail) * 4;
+    bf16_t* dst;
+    if (hh < nq) {
+      dst = q_out + ((size_t)n * nq + hh) * hd;
+    } else {
+      if (s < 0) continue;
+      dst = kc + ((page * nkv + (hh - nq)) * ps + off) * hd;
+    }
+    *reinterpret_cast<uint2*>(dst + d) = pack4(add_bias(*reinterpret_cast<const float4*>(src + hh * hd + d), hh * hd + d));
+  }
+  // values: [page][kv head][channel][slot]
+  if (s >= 0) {
+    for (int it = threadIdx.x; it < nkv * (hd / 4); it += blockDim.x) {
+      const int kvh = it / (hd / 4), d = (it - kvh * (hd / 4)) * 4, at = (nq + nkv + kvh) * hd + d;
+      const float4 v = add_bias(*reinterpret_cast<const float4*>(src + at), at);
+      bf16_t* dst = vc + ((page * nkv + kvh) * hd + d) * ps + off;
+      dst[0] = f32_to_bf16(v.x);
+      dst[(size_t)ps] = f32_to_bf16(v.y);
+      dst[(size_t)2 * ps] = f32_to_bf16(v.z);
+      dst[(size_t)3 * ps] = f32_to_bf16(v.w);
+    }
+  }
+}
+
 // cs: null, or float32 [N, rot_half, 2] from qvl_rope_table (then pos, inv_freq and freq_row are not read).
 extern "C" int qvl_rope_kv_write(const void* x, int x_stride, const void* bias, const void* pos, int pos_stride,
                                  const void* inv_freq, const void* freq_row, const void* cs, const void* slot,
@@ -221,6 +294,13 @@ extern "C" int qvl_rope_kv_write(const void* x, int x_stride, const void* bias, 
     return QVL_ERR_SHAPE;
   if (x_stride < (nq + 2 * nkv) * hd) return QVL_ERR_SHAPE;
   if (nq + 2 * nkv > 65535) return QVL_ERR_LIMIT;
+  if (in_dtype == 0 && dtype == 1 && cs && hd % 4 == 0 && rot_half % 4 == 0 && x_stride % 4 == 0 &&
+      (((uintptr_t)x | (uintptr_t)bias | (uintptr_t)cs) & 15) == 0 && (((uintptr_t)q_out | (uintptr_t)kc) & 7) == 0) {
+    hipLaunchKernelGGL(rope_kv_write_wide_kernel, dim3(N), dim3(256), 0, stream, (const float*)x, x_stride,
+                       (const float*)bias, (const float2*)cs, (const int*)slot, (bf16_t*)q_out, (bf16_t*)kc,
+                       (bf16_t*)vc, nq, nkv, hd, rot_half, ps);
+    return qvl_launch_status();
+  }
   const dim3 grid(N, nq + 2 * nkv);
 #define QVL_ROPE_CASE(ID, OD, TI, T)                                                                               \
   if (in_dtype == ID && dtype == OD) {                                                                             \

@@ -86,7 +86,12 @@ def test_rope_kv_write(dtype, nq, nkv, hd, sections):
     kc2, vc2 = torch.zeros_like(kc), torch.zeros_like(vc)
     q2 = kernels.rope_kv_write(x.cuda(), bias.cuda(), pos.to(torch.int32).cuda(), inv.cuda(), rows.cuda(), slots.cuda(),
                                kc2, vc2, nq, nkv, hd, ps, out_dtype=dtype, cs=cs)
-    assert torch.equal(q2, q) and torch.equal(kc2, kc) and torch.equal(vc2, vc)
+    if dtype == torch.float32:
+        assert torch.equal(q2, q) and torch.equal(kc2, kc) and torch.equal(vc2, vc)
+    else:   # float32 sums to bfloat16 with the table: the kernel with 16-byte loads
+        for a, b in ((q2, q), (kc2, kc), (vc2, vc)):
+            assert torch.allclose(a.float(), b.float(), atol=2e-2, rtol=1e-2)
+        assert torch.equal(vc2, vc)
     # position 0 leaves a head as it is; a negative slot writes nothing; rot < hd leaves the tail alone
     kc.zero_()
     q0 = kernels.rope_kv_write(x.cuda(), None, torch.zeros(3, n, dtype=torch.int32).cuda(), inv.cuda(), rows.cuda(),
