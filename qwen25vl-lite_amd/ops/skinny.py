@@ -46,10 +46,17 @@ def resident_norm_k() -> int:
 
 
 def takes_resident(m: int, k: int, weight: torch.Tensor, *, norm: bool = False) -> bool:
-    """Whether the resident kernel takes a product of ``m`` rows with this weight."""
+    """Whether the resident kernel takes a product of ``m`` rows with this weight, and is the
+    better choice for it.  A K that fits one pass of the block always is (the rows stay in
+    registers for all of the block's tiles).  With a longer K the rows are read again for every
+    pass of every tile, which only pays while each compute unit has a single tile (at most
+    16 weight rows each): beyond that the library's product streams such a matrix faster
+    (measured at the 72B decoder's shapes, K of 8192 and 29568)."""
     if m > RESIDENT_ROWS or k % 8 or weight.dtype != torch.bfloat16 or not _rows_aligned(weight, 8):
         return False
-    return not norm or k <= resident_norm_k()
+    if k <= resident_norm_k():
+        return True
+    return not norm and weight.shape[0] <= 16 * _compute_units(weight.device)
 
 
 def resident_product(weight: torch.Tensor, *, x: Optional[torch.Tensor] = None, h: Optional[torch.Tensor] = None,
