@@ -115,13 +115,15 @@ class CacheManager:
         """Make room for tokens ``[num_tokens, upto)`` in every group, or raise
         :class:`OutOfPages` and change nothing.  Cached prefixes nobody uses are evicted
         first if that helps."""
+        rp = self.requests[req_id]
+        if all(upto <= len(t) * self.page_size for t in rp.tables):
+            return                       # the usual case of a decoded token: its page is there
         missing = self.pages_missing(req_id, upto)
         if self.prefix_cache is not None and any(m > pool.num_free for m, pool in zip(missing, self.pools)):
             self.prefix_cache.evict(max(missing))
         for m, pool in zip(missing, self.pools):
             if m > pool.num_free:
                 raise OutOfPages(f"{m} pages wanted, {pool.num_free} free")
-        rp = self.requests[req_id]
         for g, m in enumerate(missing):
             rp.tables[g].extend(self.pools[g].allocate(m))
 

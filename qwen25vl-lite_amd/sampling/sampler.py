@@ -53,7 +53,15 @@ def sample_rows(logits: torch.Tensor, params: Sequence[SamplingParams], prev_ids
         return []
     rows = np.zeros(m, _ROW)
     flat: List[int] = []
-    for i, p in enumerate(params):
+    first = params[0]
+    if (uniforms is None and first.temperature <= 0 and first.repetition_penalty == 1.0 and first.presence_penalty == 0.0
+            and first.frequency_penalty == 0.0 and all(p is first or p == first for p in params)):
+        # one greedy setting for the whole batch (the usual decode step): fill the rows at once
+        rows[:] = (first.temperature, first.top_p, first.min_p, 0.0, 1.0, 0.0, 0.0, first.top_k if first.top_k else -1, 0, 0)
+        params_iter = ()
+    else:
+        params_iter = enumerate(params)
+    for i, p in params_iter:
         need_prev = p.repetition_penalty != 1.0 or p.presence_penalty != 0.0 or p.frequency_penalty != 0.0
         begin = len(flat)
         if need_prev:
