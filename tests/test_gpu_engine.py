@@ -59,6 +59,24 @@ def test_long_decode_and_preemption(model_dirs):
     assert llm.runner.cache.pages_in_use() == [0, 0]
 
 
+@pytest.mark.parametrize("name", ["B_sharp", "C_sharp"])
+def test_very_long_decode(model_dirs, name):
+    """Three hundred tokens decoded from a short prompt, from HIP graphs: a dozen and a half pages,
+    the window of the windowed layers passed many times over (their pages come back while the
+    request runs), several context buckets.  float32: the plain implementation's tokens."""
+    from qwen25vl_lite_amd import LLM, SamplingParams
+
+    d = model_dirs[name]
+    vocab = {"B": 509, "C": 300}[name[0]]
+    prompt = random_tokens(7, vocab, 77)
+    llm = LLM(d, dtype="float32", num_blocks=24, block_size=16, max_num_seqs=2, hip_graph=True,
+              enable_prefix_cache=False)
+    out = llm.generate([prompt], SamplingParams(temperature=0.0, max_tokens=300, ignore_eos=True))[0]
+    assert out.output_token_ids == _plain_greedy(d, prompt, 300)
+    assert len(llm.runner.graphs.graphs) >= 2
+    assert llm.runner.cache.pages_in_use() == [0] * len(llm.runner.cache.groups)
+
+
 @pytest.mark.parametrize("name, dtype", [("B_sharp", "float32"), ("C_sharp", "bfloat16"), ("A", "bfloat16")])
 def test_decode_from_hip_graphs_gives_the_same_tokens(model_dirs, name, dtype):
     """Decode steps replayed from HIP graphs, many replays with eager prefill steps, admissions and
