@@ -84,6 +84,31 @@ def test_replay_every_way(model_dirs, name, dtype):
     assert rp.runner.cache.pages_in_use() == [0] * len(rp.runner.cache.groups)
 
 
+@pytest.mark.parametrize("name, dtype", [("A_sharp", "bfloat16"), ("C", "bfloat16"), ("C_sharp", "float32"), ("A_sharp", "float32")])
+def test_long_context(model_dirs, name, dtype):
+    """More than two thousand tokens of context: the prompt in portions of 600, then single tokens,
+    whose attention splits the keys among blocks and merges the parts (bfloat16, few tiles); for
+    model C the window lies far behind the context."""
+    d = model_dirs[name]
+    vocab = VOCAB[name[0]]
+    toks = random_tokens(2160, vocab, 4242)
+    ref = _reference(d, {"long": toks}, dtype)
+    steps, n = [], 0
+    for at in range(0, 2150, 600):
+        part = toks[at:min(at + 600, 2150)]
+        steps.append({"step": n, "entries": [{"id": "long", "tokens": part, "want": [0, len(part) - 1]}], "end": []})
+        n += 1
+    for p in range(2150, 2160):
+        steps.append({"step": n, "entries": [{"id": "long", "tokens": [toks[p]], "want": [0]}],
+                      "end": ["long"] if p == 2159 else []})
+        n += 1
+    rp = _replayer(d, dtype, round64(2160))
+    got = run_steps(rp, steps)
+    assert len(got) == 2 * 4 + 10
+    print(name, dtype, "long context", _compare(got, ref, dtype, "long context"))
+    assert rp.runner.cache.pages_in_use() == [0] * len(rp.runner.cache.groups)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_explicit_position_rows(model_dirs, dtype):
     """Distinct t/h/w rows for a 4x4 block inside the prompt, then text with a rope delta
