@@ -1,4 +1,4 @@
-// Products with at most 16 rows (a decode step's projections): out[M, N] = X[M, K] . W[N, K]^T,
+// Products with at most 32 rows (a decode step's projections): out[M, N] = X[M, K] . W[N, K]^T,
 // bfloat16 operands, float32 accumulation.  The step is bound by reading W once from HBM, so W
 // is the streamed operand and everything around the product is folded into this kernel, because
 // between two products a short kernel of its own costs more than its arithmetic (its code and
@@ -10,7 +10,10 @@
 // other rows stay zero.
 // Wave w covers the 256 values of K from 256 w on, as the A operand (W rows) and B operand (X
 // rows) of v_mfma_f32_16x16x32_bf16; the 16 waves' sums meet in LDS and are added in wave order.
-// If K fits one pass (K <= 4096) the X operand stays in registers for all of the block's tiles and
+// Up to 16 rows of X are one column tile of the matrix instruction; 17 to 32 rows are two (MT = 2):
+// every W fragment that is loaded is multiplied with both.
+// If K fits one pass (K <= 4096) the X operand stays in registers (the second column tile, if
+// there is one, in LDS, which takes K <= 32 * XHI_STEPS) for all of the block's tiles and
 // the W loads of the next tile are issued before the current tile's sums are merged; a longer K is
 // walked in passes of 4096.
 //
@@ -34,6 +37,7 @@ typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 #define RW 16   // waves per block
 #define RK 8    // 32-wide K steps per wave and pass
 #define PASS_K (RW * RK * 32)
+#define XHI_STEPS 120   // 32-wide K steps of the second column tile that fit LDS beside the sums: K <= 3840
 
 enum { PRO_PLAIN = 0, PRO_NORM = 1 };
 enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2, EPI_ROPE = 3 };
@@ -79,21 +83,29 @@ __device__ __forceinline__ uint32_t pack2(float a, float b) {
   return __builtin_bit_cast(uint32_t, v);
 }
 
-template <typename TO, int PRO, int EPI, bool ONE_PASS>
+template <typename TO, int PRO, int EPI, bool ONE_PASS, int MT>
 __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) {
-  __shared__ float red[2][RW][256];   // two buffers: a tile's sums are read while the next tile's are written
+  constexpr int COLS = 16 * MT;   // rows of X the block carries
+  // MT = 1: two buffers, a tile's sums are read while the next tile's are written.  MT = 2: one
+  // (LDS also holds the second column tile of X), and the norm weights borrow it before the first tile.
+  __shared__ __attribute__((aligned(16))) float red[MT == 1 ? 2 : 1][RW][16 * COLS];
   __shared__ float rowsq[RW][16];
-  __shared__ __attribute__((aligned(16))) float gains[PRO == PRO_NORM ? RW : 1][RK * 32];   // norm weights of each wave's columns
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lg = lane >> 4, r = lane & 15;
+  __shared__ __attribute__((aligned(16))) float gains_own[(PRO == PRO_NORM && MT == 1) ? RW : 1][RK * 32];
+  __shared__ u32x4_t xhi[(MT == 2 && ONE_PASS) ? XHI_STEPS * 64 : 1];
+  float (*gains)[RK * 32] = MT == 1 ? gains_own : reinterpret_cast<float (*)[RK * 32]>(&red[0][0][0]);  // norm weights of each wave's columns
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, lg = lane >> 4, r = lane & 15;
   const int k_lane = wave * RK * 32 + 8 * lg;  // first K index of this lane within a pass
-  const bool m_ok = r < p.M;
 
   // ---- the X operand of one pass ------------------------------------------------------------
-  // first_w issues the block's first W loads at the point of the prologue where they fit best
-  auto load_x = [&](int k0, bf16x8_t* xb, auto first_w) {
+  // Column tile t holds rows 16 t .. 16 t + 15 of X.  first_w issues the block's first W loads at
+  // the point of the prologue where they fit best.  again: another column tile's norm came before
+  // (the norm weights are in LDS already, and the statistics' place may still be read).
+  auto load_x = [&](int t, int k0, bf16x8_t* xb, auto first_w, bool again = false) {
+    const int row = 16 * t + r;
+    const bool m_ok = row < p.M;
     if (PRO == PRO_PLAIN) {
       first_w();   // W first: it is the long wait
-      const bf16_t* xrow = p.X + (size_t)(m_ok ? r : 0) * p.ldx;
+      const bf16_t* xrow = p.X + (size_t)(m_ok ? row : 0) * p.ldx;
 #pragma unroll
       for (int u = 0; u < RK; ++u) {
         const int k = k0 + k_lane + u * 32;
@@ -105,7 +117,7 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
       // the norm weights are asked for first and W (by first_w) right behind them, so the
       // statistics and the scaling run while W is still on its way.  A lane fetches 4 of its
       // wave's 256 norm weights; they reach the lanes that need them through LDS.
-      const float* hrow = p.H + (size_t)(m_ok ? r : 0) * p.ldh;
+      const float* hrow = p.H + (size_t)(m_ok ? row : 0) * p.ldh;
       float4 v[RK][2];
 #pragma unroll
       for (int u = 0; u < RK; ++u) {
@@ -118,7 +130,8 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
         }
       }
       const int kg = wave * RK * 32 + 4 * lane;
-      const float4 g4 = kg < p.K ? *reinterpret_cast<const float4*>(p.norm_w + kg) : float4{0.f, 0.f, 0.f, 0.f};
+      float4 g4 = {0.f, 0.f, 0.f, 0.f};
+      if (!again && kg < p.K) g4 = *reinterpret_cast<const float4*>(p.norm_w + kg);
       first_w();
       float ss = 0.f;
 #pragma unroll
@@ -127,8 +140,9 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
               v[u][1].x * v[u][1].x + v[u][1].y * v[u][1].y + v[u][1].z * v[u][1].z + v[u][1].w * v[u][1].w;
       ss += __shfl_xor(ss, 16, QVL_WAVE);
       ss += __shfl_xor(ss, 32, QVL_WAVE);
+      if (again) __syncthreads();   // the other column tile's statistics have been read
       if (lg == 0) rowsq[wave][r] = ss;
-      *reinterpret_cast<float4*>(&gains[wave][4 * lane]) = g4;
+      if (!again) *reinterpret_cast<float4*>(&gains[wave][4 * lane]) = g4;
       __syncthreads();
       float total = 0.f;
 #pragma unroll
@@ -168,16 +182,18 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
     }
     return tile * p.rows + i;
   };
-  auto load_w = [&](int tile, int k0, bf16x8_t* a) {
+  // steps u0 .. u0 + n - 1 of a tile's W operand
+  auto load_w_part = [&](int tile, int k0, int u0, int n, bf16x8_t* a) {
     const int row = w_row(tile, r);
     const bool row_ok = r < tile_rows(tile) && row >= 0 && row < p.N;
     const bf16_t* wrow = p.W + (size_t)(row_ok ? row : 0) * p.ldw;
 #pragma unroll
-    for (int u = 0; u < RK; ++u) {
-      const int k = k0 + k_lane + u * 32;
+    for (int u = 0; u < n; ++u) {
+      const int k = k0 + k_lane + (u0 + u) * 32;
       a[u] = (row_ok && k < p.K) ? load8(wrow + k) : zero8();
     }
   };
+  auto load_w = [&](int tile, int k0, bf16x8_t* a) { load_w_part(tile, k0, 0, RK, a); };
   // What the epilogue of a tile reads from memory, for the element (m, nl) this thread finishes.
   // Loads return in the order they are issued, so these are asked for before the W loads of the
   // next tile: waiting for them must not wait for those.
@@ -191,7 +207,7 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
     e.bias = e.old = 0.f;
     e.cs = float2{1.f, 0.f};
     e.slot = -1;
-    if (threadIdx.x >= 256 || EPI == EPI_SWIGLU) return e;
+    if (threadIdx.x >= 16 * COLS || EPI == EPI_SWIGLU) return e;
     const int m = threadIdx.x >> 4, nl = threadIdx.x & 15, n = w_row(tile, nl);
     if (m >= p.M || nl >= tile_rows(tile) || n >= p.N) return e;
     if (p.bias) e.bias = p.bias[n];
@@ -205,21 +221,27 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
     return e;
   };
   // ---- merge the waves' sums of one tile and write the result -----------------------------------
-  // One barrier per tile: the sums go into the buffer that was read two tiles ago; whoever reads
-  // it (the first four waves) has passed the barrier of the tile in between since.
+  // A wave's sums lie as [row of X][row of the tile]: a lane writes its four at once, and the
+  // thread that finishes element e = 16 m + nl reads word e of every wave.
+  // MT = 1, one barrier per tile: the sums go into the buffer that was read two tiles ago; whoever
+  // reads it (the first four waves) has passed the barrier of the tile in between since.
+  // MT = 2, one buffer: a second barrier keeps the next tile's sums out until these are read.
+  struct Acc {
+    f32x4_t t[MT];
+  };
   int parity = 0;
-  auto finish = [&](int tile, const f32x4_t& acc, const Epi& epi) {
-    float (*buf)[256] = red[parity];
+  auto finish = [&](int tile, const Acc& acc, const Epi& epi) {
+    float (*buf)[16 * COLS] = red[MT == 1 ? parity : 0];
     parity ^= 1;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) buf[wave][(4 * lg + i) * 16 + r] = acc[i];
+    for (int t = 0; t < MT; ++t) *reinterpret_cast<f32x4_t*>(&buf[wave][(16 * t + r) * 16 + 4 * lg]) = acc.t[t];
     __syncthreads();
-    if (threadIdx.x < 256) {
+    if (threadIdx.x < 16 * COLS) {
       const int e = threadIdx.x;
       const int m = e >> 4, nl = e & 15, n = w_row(tile, nl);
       float sum = 0.f;
 #pragma unroll
-      for (int w = 0; w < RW; ++w) sum += buf[w][nl * 16 + m];
+      for (int w = 0; w < RW; ++w) sum += buf[w][e];
       if (EPI == EPI_SWIGLU) {
         const float up = __shfl_down(sum, 8, QVL_WAVE);  // rows 8..15 of the tile are the up rows
         if (nl < 8 && m < p.M && n >= 0 && n < p.N) {
@@ -254,37 +276,83 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
         }
       }
     }
+    if (MT == 2) __syncthreads();
   };
-  auto product = [&](const bf16x8_t* a, const bf16x8_t* xb, f32x4_t acc) {
+  // The W operand's steps come as two halves (a_lo, a_hi).  x1: the second column tile's operand in
+  // registers; null: it is in LDS (one pass), except for the waves whose steps lie beyond K then.
+  const bool hi_live = wave * RK < XHI_STEPS;
+  auto product = [&](const bf16x8_t* a_lo, const bf16x8_t* a_hi, const bf16x8_t* x0, const bf16x8_t* x1, Acc acc) {
 #pragma unroll
-    for (int u = 0; u < RK; ++u) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], xb[u], acc, 0, 0, 0);
+    for (int u = 0; u < RK; ++u) {
+      const bf16x8_t a = u < RK / 2 ? a_lo[u] : a_hi[u - RK / 2];
+      acc.t[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, x0[u], acc.t[0], 0, 0, 0);
+      if (MT == 2) {
+        if (!ONE_PASS)
+          acc.t[MT - 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, x1[u], acc.t[MT - 1], 0, 0, 0);
+        else if (hi_live)
+          acc.t[MT - 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+              a, __builtin_bit_cast(bf16x8_t, xhi[(wave * RK + u) * 64 + lane]), acc.t[MT - 1], 0, 0, 0);
+      }
+    }
     return acc;
   };
-  const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
+  Acc zero;
+#pragma unroll
+  for (int t = 0; t < MT; ++t) zero.t[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
   if (ONE_PASS) {
+    // Three half-tile buffers of W go round: while a tile is multiplied, the first half of the next
+    // is on its way; its second half and the first half of the tile after it are asked for as soon
+    // as the product has freed their registers, and arrive during the merge of the sums.
     bf16x8_t xb[RK];
-    bf16x8_t a[2][RK];
+    bf16x8_t w[3][RK / 2];
     int tile = blockIdx.x;
-    load_x(0, xb, [&] { if (tile < p.ntiles) load_w(tile, 0, a[0]); });
-    for (; tile < p.ntiles; tile += 2 * gridDim.x) {
-      const int t1 = tile + gridDim.x, t2 = tile + 2 * gridDim.x;
-      const Epi e0 = epi_load(tile);
-      if (t1 < p.ntiles) load_w(t1, 0, a[1]);
-      finish(tile, product(a[0], xb, zero), e0);
-      if (t1 >= p.ntiles) break;
-      const Epi e1 = epi_load(t1);
-      if (t2 < p.ntiles) load_w(t2, 0, a[0]);
-      finish(t1, product(a[1], xb, zero), e1);
+    if (MT == 1) {
+      load_x(0, 0, xb, [&] {
+        if (tile < p.ntiles) {
+          load_w_part(tile, 0, 0, RK / 2, w[0]);
+          load_w_part(tile, 0, RK / 2, RK / 2, w[1]);
+        }
+      });
+    } else {
+      // rows 16..31 first, while few registers are taken: each lane keeps its own operands of
+      // them in LDS and reads them back itself
+      bf16x8_t hi[RK];
+      load_x(1, 0, hi, [&] { if (tile < p.ntiles) load_w_part(tile, 0, 0, RK / 2, w[0]); });
+#pragma unroll
+      for (int u = 0; u < RK; ++u)
+        if (hi_live) xhi[(wave * RK + u) * 64 + lane] = __builtin_bit_cast(u32x4_t, hi[u]);
+      load_x(0, 0, xb, [&] { if (tile < p.ntiles) load_w_part(tile, 0, RK / 2, RK / 2, w[1]); }, true);
+      if (PRO == PRO_NORM) __syncthreads();   // the norm weights lie where the first tile's sums go
+    }
+    Epi e = epi_load(tile);
+    if (tile + gridDim.x < p.ntiles) load_w_part(tile + gridDim.x, 0, 0, RK / 2, w[2]);
+    // one tile whose halves are in a_lo and a_hi; false: it was the block's last
+    auto one = [&](bf16x8_t* a_lo, bf16x8_t* a_hi) {
+      const Acc acc = product(a_lo, a_hi, xb, nullptr, zero);
+      const int next = tile + gridDim.x, after = next + gridDim.x;
+      const Epi e_next = epi_load(next);
+      if (next < p.ntiles) load_w_part(next, 0, RK / 2, RK / 2, a_lo);
+      if (after < p.ntiles) load_w_part(after, 0, 0, RK / 2, a_hi);
+      finish(tile, acc, e);
+      e = e_next;
+      tile = next;
+      return next < p.ntiles;
+    };
+    while (tile < p.ntiles) {
+      if (!one(w[0], w[1])) break;
+      if (!one(w[2], w[0])) break;
+      if (!one(w[1], w[2])) break;
     }
   } else {
     for (int tile = blockIdx.x; tile < p.ntiles; tile += gridDim.x) {
-      f32x4_t acc = zero;
+      Acc acc = zero;
       const Epi e = epi_load(tile);
       for (int k0 = 0; k0 < p.K; k0 += PASS_K) {
-        bf16x8_t xb[RK], a[RK];
-        load_x(k0, xb, [&] { load_w(tile, k0, a); });
-        acc = product(a, xb, acc);
+        bf16x8_t xb[RK], x1[MT == 2 ? RK : 1], a[RK];
+        load_x(0, k0, xb, [&] { load_w(tile, k0, a); });
+        if (MT == 2) load_x(1, k0, x1, [] {}, true);
+        acc = product(a, a + RK / 2, xb, x1, acc);
       }
       finish(tile, acc, e);
     }
@@ -294,13 +362,19 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
 template <typename TO, int PRO, int EPI>
 static void launch(const ResidentArgs& p, int blocks, hipStream_t stream) {
   const dim3 grid(blocks < p.ntiles ? blocks : p.ntiles), block(64 * RW);
-  if (p.K <= PASS_K)
-    hipLaunchKernelGGL((gemm_resident_kernel<TO, PRO, EPI, true>), grid, block, 0, stream, p);
+  if (p.K <= PASS_K && p.M <= 16)
+    hipLaunchKernelGGL((gemm_resident_kernel<TO, PRO, EPI, true, 1>), grid, block, 0, stream, p);
+  else if (p.K <= 32 * XHI_STEPS)
+    hipLaunchKernelGGL((gemm_resident_kernel<TO, PRO, EPI, true, 2>), grid, block, 0, stream, p);
+  else if (p.M <= 16)
+    hipLaunchKernelGGL((gemm_resident_kernel<TO, PRO, EPI, false, 1>), grid, block, 0, stream, p);
   else
-    hipLaunchKernelGGL((gemm_resident_kernel<TO, PRO, EPI, false>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((gemm_resident_kernel<TO, PRO, EPI, false, 2>), grid, block, 0, stream, p);
 }
 
 extern "C" int qvl_gemm_resident_pass_k() { return PASS_K; }
+// the longest K with which 17 to 32 rows stay resident (and with which their norm is folded in)
+extern "C" int qvl_gemm_resident_two_tile_k() { return 32 * XHI_STEPS; }
 
 // x: bfloat16 [M, K] (h null), or h: float32 [M, K] with norm_w [K] and eps (x null): X = rmsnorm(h) * norm_w.
 // epilogue 0: out[M, N] in out_dtype (0 float32, 1 bfloat16); 1: out (float32 [M, N]) += product;
@@ -310,11 +384,12 @@ extern "C" int qvl_gemm_resident(const void* x, int ldx, const void* h, int ldh,
                                  const void* W, int ldw, const void* bias, void* out, int ldo, int M, int N, int K,
                                  int out_dtype, int epilogue, int max_blocks, hipStream_t stream) {
   if (M <= 0 || N <= 0) return QVL_OK;
-  if (M > 16) return QVL_ERR_LIMIT;
+  if (M > 32) return QVL_ERR_LIMIT;
   if (K <= 0 || K % 8 || ldw % 8 || ldw < K || max_blocks <= 0 || !W || !out) return QVL_ERR_SHAPE;
   const bool norm = h != nullptr;
   if (norm) {
     if (x || !norm_w || K > PASS_K || ldh % 4 || ldh < K) return QVL_ERR_SHAPE;
+    if (M > 16 && K > 32 * XHI_STEPS) return QVL_ERR_LIMIT;
   } else if (!x || ldx % 8 || ldx < K) {
     return QVL_ERR_SHAPE;
   }
@@ -361,7 +436,7 @@ extern "C" int qvl_gemm_resident(const void* x, int ldx, const void* h, int ldh,
   return qvl_launch_status();
 }
 
-// The stacked query | key | value projection of at most 16 tokens with rotation and cache write
+// The stacked query | key | value projection of at most 32 tokens with rotation and cache write
 // folded in (EPI_ROPE).  x / h / norm_w / eps as in qvl_gemm_resident.  W: [(nq + 2 nkv) hd, K];
 // bias: float32 [(nq + 2 nkv) hd] or null.  cs: float32 [M, hd / 2, 2], cosine and sine of every
 // token's angle at every frequency (1 and 0 where a frequency is not rotated);
@@ -373,13 +448,14 @@ extern "C" int qvl_gemm_resident_rope(const void* x, int ldx, const void* h, int
                                       const void* slot, void* q_out, void* kc, void* vc, int nq, int nkv, int hd, int ps,
                                       int max_blocks, hipStream_t stream) {
   if (M <= 0) return QVL_OK;
-  if (M > 16) return QVL_ERR_LIMIT;
+  if (M > 32) return QVL_ERR_LIMIT;
   if (K <= 0 || K % 8 || ldw % 8 || ldw < K || max_blocks <= 0 || !W || !q_out) return QVL_ERR_SHAPE;
   if (nq <= 0 || nkv < 0 || hd <= 0 || hd % 16 || ps <= 0 || !cs) return QVL_ERR_SHAPE;
   if (nkv > 0 && (!slot || !kc || !vc)) return QVL_ERR_SHAPE;
   const bool norm = h != nullptr;
   if (norm) {
     if (x || !norm_w || K > PASS_K || ldh % 4 || ldh < K) return QVL_ERR_SHAPE;
+    if (M > 16 && K > 32 * XHI_STEPS) return QVL_ERR_LIMIT;
   } else if (!x || ldx % 8 || ldx < K) {
     return QVL_ERR_SHAPE;
   }

@@ -1,8 +1,9 @@
 """Dispatch of bfloat16 products with few rows to the hand-written kernels.
 
-Up to 16 rows: the resident kernel (``csrc/gemm_resident.hip``), which can also fold the RMSNorm
-before the product, the residual add after it, or the SwiGLU activation into itself.
-17 to 32 rows: the streaming kernel (``csrc/gemm_skinny.hip``) where it beats the library.
+Up to 32 rows: the resident kernel (``csrc/gemm_resident.hip``), which can also fold the RMSNorm
+before the product, the residual add after it, or the SwiGLU activation into itself; with 17 to 32
+rows it needs an inner size that fits one pass of a block.
+17 to 32 rows beyond that: the streaming kernel (``csrc/gemm_skinny.hip``) where it beats the library.
 """
 
 from __future__ import annotations
@@ -14,12 +15,13 @@ import torch
 
 from .kernels import _check, _fn, _ptr, _stream, dtype_code
 
-__all__ = ["resident_product", "takes_resident", "qkv_rope_product", "takes_qkv_rope", "try_streaming", "RESIDENT_ROWS", "resident_norm_k", "MAX_ROWS",
+__all__ = ["resident_product", "takes_resident", "qkv_rope_product", "takes_qkv_rope", "try_streaming", "RESIDENT_ROWS", "resident_norm_k", "resident_two_tile_k", "folds_norm", "MAX_ROWS",
            "STORE", "RESIDUAL", "SWIGLU"]
 
 MAX_ROWS = 32            # the streaming kernel's limit in use
-RESIDENT_ROWS = 16       # up to here the resident kernel runs
+RESIDENT_ROWS = 32       # up to here the resident kernel runs (one column tile of 16 rows, or two)
 _pass_k = None
+_two_tile_k = None
 STORE, RESIDUAL, SWIGLU = 0, 1, 2
 _c_int, _c_float, _c_ptr = ctypes.c_int, ctypes.c_float, ctypes.c_void_p
 _cu_count = {}
@@ -45,6 +47,20 @@ def resident_norm_k() -> int:
     return _pass_k
 
 
+def resident_two_tile_k() -> int:
+    """The longest inner size with which the resident kernel takes 17 to 32 rows (their second
+    half waits in LDS; the kernel's own constant)."""
+    global _two_tile_k
+    if _two_tile_k is None:
+        _two_tile_k = int(_fn("gemm_resident", "qvl_gemm_resident_two_tile_k", [])())
+    return _two_tile_k
+
+
+def folds_norm(m: int, k: int) -> bool:
+    """Whether the resident kernel forms the norm of ``m`` rows of width ``k`` by itself."""
+    return m <= RESIDENT_ROWS and k <= (resident_norm_k() if m <= 16 else resident_two_tile_k())
+
+
 def takes_resident(m: int, k: int, weight: torch.Tensor, *, norm: bool = False) -> bool:
     """Whether the resident kernel takes a product of ``m`` rows with this weight, and is the
     better choice for it.  A K that fits one pass of the block always is (the rows stay in
@@ -54,7 +70,7 @@ def takes_resident(m: int, k: int, weight: torch.Tensor, *, norm: bool = False) 
     (measured at the 72B decoder's shapes, K of 8192 and 29568)."""
     if m > RESIDENT_ROWS or k % 8 or weight.dtype != torch.bfloat16 or not _rows_aligned(weight, 8):
         return False
-    if k <= resident_norm_k():
+    if k <= (resident_norm_k() if m <= 16 else resident_two_tile_k()):
         return True
     return not norm and weight.shape[0] <= 16 * _compute_units(weight.device)
 
@@ -63,7 +79,7 @@ def resident_product(weight: torch.Tensor, *, x: Optional[torch.Tensor] = None, 
                      norm_weight: Optional[torch.Tensor] = None, eps: float = 0.0,
                      bias: Optional[torch.Tensor] = None, epilogue: int = STORE,
                      out: Optional[torch.Tensor] = None, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
-    """``X @ weight.T`` for at most 16 rows.  ``X`` is ``x`` (bfloat16), or ``rmsnorm(h) * norm_weight``
+    """``X @ weight.T`` for at most 32 rows.  ``X`` is ``x`` (bfloat16), or ``rmsnorm(h) * norm_weight``
     formed inside the kernel from the float32 rows ``h``.  ``epilogue``: ``STORE`` writes the product
     (plus ``bias``) to a new tensor of ``out_dtype``; ``RESIDUAL`` adds it to ``out`` (float32) in
     place; ``SWIGLU`` takes ``weight``'s rows as groups of 8 gate, 8 up rows and returns
@@ -112,7 +128,7 @@ def qkv_rope_product(weight: torch.Tensor, cs: torch.Tensor, *, x: Optional[torc
                      bias: Optional[torch.Tensor] = None, slots: Optional[torch.Tensor] = None,
                      k_cache: Optional[torch.Tensor] = None, v_cache: Optional[torch.Tensor] = None,
                      num_q_heads: int, num_kv_heads: int, head_dim: int, page_size: int) -> torch.Tensor:
-    """The stacked query | key | value projection of at most 16 tokens with the rotation and the
+    """The stacked query | key | value projection of at most 32 tokens with the rotation and the
     cache write inside the product's kernel: returns the rotated queries ``[M, nq hd]`` (bfloat16);
     rotated keys and values are in their page slots.  ``cs`` is :func:`kernels.rope_table` of the
     step's tokens.  With ``num_kv_heads == 0`` the weight holds query rows only."""
@@ -154,7 +170,7 @@ def prefers_streaming(m: int, n: int, k: int) -> bool:
     """Where the streaming kernel (rows of x read again from L2 by every wave) beats the library's
     product on MI355X, measured at the 7B decoder's shapes with 17 to 32 rows: the small square
     matrix and the one with a long inner size."""
-    return RESIDENT_ROWS < m <= MAX_ROWS and (n * k <= 13_000_000 or k >= 4 * n)
+    return 16 < m <= MAX_ROWS and (n * k <= 13_000_000 or k >= 4 * n)
 
 
 def try_streaming(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
