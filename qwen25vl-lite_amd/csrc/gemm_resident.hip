@@ -300,13 +300,22 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
 #pragma unroll
   for (int t = 0; t < MT; ++t) zero.t[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-  if (ONE_PASS) {
-    // Three half-tile buffers of W go round: while a tile is multiplied, the first half of the next
-    // is on its way; its second half and the first half of the tile after it are asked for as soon
-    // as the product has freed their registers, and arrive during the merge of the sums.
+  if (ONE_PASS || MT == 1) {
+    // The block's work is a sequence of steps: every tile of its own, and within a tile every pass
+    // over K (one, if X stays resident).  Three half-step buffers of W go round: while a step is
+    // multiplied, the first half of the next is on its way; its second half and the first half of
+    // the step after it are asked for as soon as the product has freed their registers, and arrive
+    // during the merge of the sums (or, between the passes of a tile, while the next rows of X come).
+    const int passes = ONE_PASS ? 1 : (p.K + PASS_K - 1) / PASS_K;
+    auto step_after = [&](int& t, int& ps) {
+      if (++ps >= passes) {
+        ps = 0;
+        t += gridDim.x;
+      }
+    };
     bf16x8_t xb[RK];
     bf16x8_t w[3][RK / 2];
-    int tile = blockIdx.x;
+    int tile = blockIdx.x, pass = 0;
     if (MT == 1) {
       load_x(0, 0, xb, [&] {
         if (tile < p.ntiles) {
@@ -326,18 +335,35 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
       if (PRO == PRO_NORM) __syncthreads();   // the norm weights lie where the first tile's sums go
     }
     Epi e = epi_load(tile);
-    if (tile + gridDim.x < p.ntiles) load_w_part(tile + gridDim.x, 0, 0, RK / 2, w[2]);
-    // one tile whose halves are in a_lo and a_hi; false: it was the block's last
+    {
+      int t1 = tile, p1 = 0;
+      step_after(t1, p1);
+      if (t1 < p.ntiles) load_w_part(t1, p1 * PASS_K, 0, RK / 2, w[2]);
+    }
+    Acc acc = zero;
+    // one step whose halves are in a_lo and a_hi; false: it was the block's last
     auto one = [&](bf16x8_t* a_lo, bf16x8_t* a_hi) {
-      const Acc acc = product(a_lo, a_hi, xb, nullptr, zero);
-      const int next = tile + gridDim.x, after = next + gridDim.x;
-      const Epi e_next = epi_load(next);
-      if (next < p.ntiles) load_w_part(next, 0, RK / 2, RK / 2, a_lo);
-      if (after < p.ntiles) load_w_part(after, 0, 0, RK / 2, a_hi);
-      finish(tile, acc, e);
-      e = e_next;
-      tile = next;
-      return next < p.ntiles;
+      acc = product(a_lo, a_hi, xb, nullptr, acc);
+      int tn = tile, pn = pass;
+      step_after(tn, pn);
+      int ta = tn, pa = pn;
+      step_after(ta, pa);
+      const bool tile_done = ONE_PASS || pn == 0;
+      Epi e_next = e;
+      if (tile_done) e_next = epi_load(tn);
+      if (tn < p.ntiles) {
+        if (!ONE_PASS) load_x(0, pn * PASS_K, xb, [] {});
+        load_w_part(tn, pn * PASS_K, RK / 2, RK / 2, a_lo);
+      }
+      if (ta < p.ntiles) load_w_part(ta, pa * PASS_K, 0, RK / 2, a_hi);
+      if (tile_done) {
+        finish(tile, acc, e);
+        acc = zero;
+        e = e_next;
+      }
+      tile = tn;
+      pass = pn;
+      return tn < p.ntiles;
     };
     while (tile < p.ntiles) {
       if (!one(w[0], w[1])) break;
@@ -366,10 +392,12 @@ static void launch(const ResidentArgs& p, int blocks, hipStream_t stream) {
     hipLaunchKernelGGL((gemm_resident_kernel<TO, PRO, EPI, true, 1>), grid, block, 0, stream, p);
   else if (p.K <= 32 * XHI_STEPS)
     hipLaunchKernelGGL((gemm_resident_kernel<TO, PRO, EPI, true, 2>), grid, block, 0, stream, p);
-  else if (p.M <= 16)
-    hipLaunchKernelGGL((gemm_resident_kernel<TO, PRO, EPI, false, 1>), grid, block, 0, stream, p);
-  else
-    hipLaunchKernelGGL((gemm_resident_kernel<TO, PRO, EPI, false, 2>), grid, block, 0, stream, p);
+  else if constexpr (PRO == PRO_PLAIN) {   // a norm is only folded into a single pass: the host has checked
+    if (p.M <= 16)
+      hipLaunchKernelGGL((gemm_resident_kernel<TO, PRO, EPI, false, 1>), grid, block, 0, stream, p);
+    else
+      hipLaunchKernelGGL((gemm_resident_kernel<TO, PRO, EPI, false, 2>), grid, block, 0, stream, p);
+  }
 }
 
 extern "C" int qvl_gemm_resident_pass_k() { return PASS_K; }

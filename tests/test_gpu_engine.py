@@ -123,6 +123,42 @@ def test_decode_graphs_with_padding_rows(model_dirs, name, dtype):
     assert llm.runner.cache.pages_in_use() == [0] * len(llm.runner.cache.groups)
 
 
+@pytest.mark.parametrize("name, hip_graph", [("C_sharp", False), ("B_sharp", True)])
+def test_twenty_odd_requests_decode_together(model_dirs, name, hip_graph):
+    """Between 17 and 32 decoded tokens a step the bfloat16 products run with two column tiles of
+    rows (norm, rotation with cache write, activation and residual folded in as with fewer): 21
+    requests of different lengths, some ending early so that the batch shrinks through 24, 16 and
+    12 rows.  float32 gives the plain implementation's tokens.  bfloat16 gives them up to the first
+    place where the plain logits' two best lie closer than the bound on bfloat16 logits (2e-2, as
+    in the replay tests): there either token is right, and what follows it is another sequence."""
+    from qwen25vl_lite_amd import LLM, SamplingParams
+
+    d = model_dirs[name]
+    vocab = {"B": 509, "C": 300}[name[0]]
+    prompts = [random_tokens(3 + (5 * i) % 23, vocab, 300 + i) for i in range(21)]
+    params = [SamplingParams(temperature=0.0, max_tokens=4 + (7 * i) % 19, ignore_eos=True) for i in range(21)]
+    common = dict(num_blocks=128, block_size=16, max_num_seqs=32, max_num_batched_tokens=512,
+                  enable_prefix_cache=False, hip_graph=hip_graph)
+    exact = LLM(d, dtype="float32", **common).generate(prompts, params)
+    llm = LLM(d, dtype="bfloat16", **common)
+    outs = llm.generate(prompts, params)
+    if hip_graph:
+        assert 24 in {k[0] for k in llm.runner.graphs.graphs}
+    whole = 0
+    for prompt, out, ex, p in zip(prompts, outs, exact, params):
+        want = _plain_greedy(d, prompt, p.max_tokens)
+        assert ex.output_token_ids == want
+        got = out.output_token_ids
+        if got == want:
+            whole += 1
+            continue
+        j = next(k for k in range(len(want)) if got[k] != want[k])
+        best = torch.topk(plain_model_logits(d, list(prompt) + want[:j])[-1], 2)
+        assert got[j] == int(best.indices[1]) and float(best.values[0] - best.values[1]) < 2e-2, (j, best)
+    assert whole >= 14          # ties are the exception
+    assert llm.runner.cache.pages_in_use() == [0] * len(llm.runner.cache.groups)
+
+
 @pytest.mark.parametrize("name, seed", [("A_sharp", 0), ("A_sharp", 1), ("C_sharp", 2)])
 def test_everything_at_once(model_dirs, name, seed):
     """A server's day in small: requests of random lengths, some sharing a prefix, more of them than
