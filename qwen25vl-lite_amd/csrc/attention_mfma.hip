@@ -321,11 +321,20 @@ __device__ __forceinline__ void init_state(TileState& st) {
 // No register holds data in flight, so BLK_STAGES - 1 blocks are on their way while one is
 // computed.  The loads are issued from inline assembly and waited for with explicit vmcnt values:
 // every wave issues exactly WAVE_LOADS of them per block.
+// With head sizes up to 128 the kernel also comes with GROUPS = 2 such groups of BLK_WAVES waves in
+// a workgroup, on the same column tiles: group g walks the key blocks g, g + 2, ... through stages
+// of its own, and the groups' sums are merged through LDS at the end.  One such workgroup fills a
+// compute unit where two of the plain kind do, and a walk takes half as long.  That pays where a
+// step has no more walks than the plain kind has places and they differ much in length (one
+// prompt of 2,048 tokens: the first tiles see few keys, the last ones all); with more walks the
+// plain kind's independent workgroups overlap their matrix and vector phases better.
 #define BLK_WAVES 4
 #if HD <= 128
 #define BLK_CT 2
+#define BLK_MAX_GROUPS 2
 #else
 #define BLK_CT 1
+#define BLK_MAX_GROUPS 1
 #endif
 #define BLK_STAGES 4
 #define CH_PER_KEY (HD / 8)                                       // 16-byte chunks of a key
@@ -362,7 +371,8 @@ struct StagePages {
 // q / (CH_PER_KEY + 1), slot q of V^T is keys 8 (q mod 5) .. + 7 of channel q / 5.  Everything
 // about a lane's address that does not change from block to block is worked out once (start);
 // the halves' page index and slot move along with the blocks (next_pages is called for
-// consecutive blocks), so the page size is divided by once.
+// the blocks kb, kb + GROUPS, ... of a group), so the page size is divided by once.
+template <int GROUPS>
 struct BlockLoader {
   const bf16_t* kc;
   const bf16_t* vc;
@@ -414,9 +424,9 @@ struct BlockLoader {
       const int p = idx[h] < table_width ? bt[idx[h]] : 0;
       pg.page[h] = p < 0 ? 0 : p;
       pg.off[h] = off[h];
-      off[h] += 32;  // a page has at least 16 slots: at most two pages further
+      off[h] += 32 * GROUPS;  // the group's next block; a page has at least 16 slots
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < 2 * GROUPS; ++i)
         if (off[h] >= ps) {
           off[h] -= ps;
           ++idx[h];
@@ -458,13 +468,19 @@ __device__ __forceinline__ void operands_from_lds(const bf16_t* ks, const bf16_t
 
 // One entry of the block list for one key/value head.  blk_cb counts in units of
 // BLK_WAVES * BLK_CT column tiles.
+template <int GROUPS>
 struct BlockShared {
-  __attribute__((aligned(16))) bf16_t stage[BLK_STAGES][STAGE_ELEMS];   // K rows, then V^T rows
-  int wave_range[BLK_WAVES][2];
+  __attribute__((aligned(16))) bf16_t stage[GROUPS][BLK_STAGES][STAGE_ELEMS];   // K rows, then V^T rows
+  int wave_range[GROUPS * BLK_WAVES][2];
   int work;
 };
+// what a lane of the second group hands over per column tile: its sums, the reference and its share of the total
+#define MERGE_REGS (NT * 4 + 2)
+static_assert(BLK_MAX_GROUPS == 1 || BLK_CT * MERGE_REGS * BLK_WAVES * 64 * 4 <= BLK_STAGES * STAGE_ELEMS * 2,
+              "the second group's sums do not fit its stages");
 
-__device__ __forceinline__ void attend_block(BlockShared& sh, int item, int kvh, const bf16_t* __restrict__ q,
+template <int GROUPS>
+__device__ __forceinline__ void attend_block(BlockShared<GROUPS>& sh, int item, int kvh, const bf16_t* __restrict__ q,
                                              const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
                                              const int* __restrict__ bt, int table_width,
                                              const int* __restrict__ cu_q, const int* __restrict__ ctx_len,
@@ -472,7 +488,8 @@ __device__ __forceinline__ void attend_block(BlockShared& sh, int item, int kvh,
                                              bf16_t* __restrict__ out, int nq, int nkv, int ps, int window,
                                              float scale) {
   const int g = nq / nkv;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int wave_of_all = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int group = wave_of_all / BLK_WAVES, wave = wave_of_all % BLK_WAVES;
   const int r = blk_req[item], ct0 = (blk_cb[item] * BLK_WAVES + wave) * BLK_CT;
   const int ncols = (cu_q[r + 1] - cu_q[r]) * g;
   TileInfo t[BLK_CT];
@@ -495,13 +512,13 @@ __device__ __forceinline__ void attend_block(BlockShared& sh, int item, int kvh,
     }
   }
   if (lane == 0) {
-    sh.wave_range[wave][0] = lo;
-    sh.wave_range[wave][1] = hi;
+    sh.wave_range[wave_of_all][0] = lo;
+    sh.wave_range[wave_of_all][1] = hi;
   }
   __syncthreads();
   int blo = 0x7fffffff, bhi = -1;
 #pragma unroll
-  for (int i = 0; i < BLK_WAVES; ++i) {
+  for (int i = 0; i < GROUPS * BLK_WAVES; ++i) {
     blo = min(blo, sh.wave_range[i][0]);
     bhi = max(bhi, sh.wave_range[i][1]);
   }
@@ -526,11 +543,15 @@ __device__ __forceinline__ void attend_block(BlockShared& sh, int item, int kvh,
     w.all_lo = a;
     w.all_hi = b;
   }
-  BlockLoader ld;
+  BlockLoader<GROUPS> ld;
   ld.kc = kc; ld.vc = vc; ld.bt = bt + (size_t)r * table_width;
   ld.table_width = table_width; ld.ps = ps; ld.wave = wave;
-  const int kb0 = blo >> 5, nblk = (bhi >> 5) - kb0 + 1;
-  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)&sh.stage[0][0];
+  // this group's blocks are kb0, kb0 + GROUPS, ...: nblk of them; every group goes round the
+  // loop (and through its barrier) as often as the first
+  const int kb0 = (blo >> 5) + group, all_blocks = (bhi >> 5) - (blo >> 5) + 1;
+  const int nblk = (all_blocks - group + GROUPS - 1) / GROUPS;
+  const int rounds = (all_blocks + GROUPS - 1) / GROUPS;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)&sh.stage[group][0][0];
   StagePages pg;
   ld.start(kb0, nkv, kvh);
   ld.next_pages(pg);
@@ -545,7 +566,7 @@ __device__ __forceinline__ void attend_block(BlockShared& sh, int item, int kvh,
       ++issued;
       if (issued < nblk) ld.next_pages(pg);
     }
-  for (int i = 0; i < nblk; ++i) {
+  for (int i = 0; i < rounds; ++i) {
     // block i has landed when only the loads of the blocks issued after it are outstanding
     const int later = issued - 1 - i;
     if (later >= 2) wait_loads<2 * WAVE_LOADS>();
@@ -557,12 +578,46 @@ __device__ __forceinline__ void attend_block(BlockShared& sh, int item, int kvh,
       ++issued;
       if (issued < nblk) ld.next_pages(pg);
     }
-    const int kb = kb0 + i;
-    if ((kb << 5) + 31 >= lo && (kb << 5) <= hi) {
-      const bf16_t* stage = sh.stage[i % BLK_STAGES];
+    const int kb = kb0 + GROUPS * i;
+    if (i < nblk && (kb << 5) + 31 >= lo && (kb << 5) <= hi) {
+      const bf16_t* stage = sh.stage[group][i % BLK_STAGES];
       BlockRegs ops;
       operands_from_lds(stage, stage + K_LOADS * 512, ops);
       w.compute(kb, qb, ops, st);
+    }
+  }
+  if (GROUPS > 1) {
+    // The second group's sums reach the first through the second group's stages, which nobody reads
+    // or fills any more: word (tile, register, wave, lane), so every lane finds its partner's.
+    float* hand = reinterpret_cast<float*>(&sh.stage[GROUPS - 1][0][0]);
+    __syncthreads();
+    if (group > 0) {
+#pragma unroll
+      for (int i = 0; i < BLK_CT; ++i) {
+        float* mine = hand + ((size_t)i * MERGE_REGS * BLK_WAVES + wave) * 64 + lane;
+#pragma unroll
+        for (int dt = 0; dt < NT; ++dt)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) mine[(dt * 4 + j) * BLK_WAVES * 64] = st[i].acc[dt][j];
+        mine[(NT * 4) * BLK_WAVES * 64] = st[i].m;
+        mine[(NT * 4 + 1) * BLK_WAVES * 64] = st[i].l;
+      }
+    }
+    __syncthreads();
+    if (group > 0) return;
+#pragma unroll
+    for (int i = 0; i < BLK_CT; ++i) {
+      const float* theirs = hand + ((size_t)i * MERGE_REGS * BLK_WAVES + wave) * 64 + lane;
+      const float m_b = theirs[(NT * 4) * BLK_WAVES * 64], l_b = theirs[(NT * 4 + 1) * BLK_WAVES * 64];
+      const float m = fmaxf(st[i].m, m_b);
+      const float ref = m == -INFINITY ? 0.f : m;   // a column without keys: both sides are zero
+      const float sa = __builtin_amdgcn_exp2f(st[i].m - ref), sb = __builtin_amdgcn_exp2f(m_b - ref);
+      st[i].l = st[i].l * sa + l_b * sb;
+#pragma unroll
+      for (int dt = 0; dt < NT; ++dt)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          st[i].acc[dt][j] = st[i].acc[dt][j] * sa + theirs[(dt * 4 + j) * BLK_WAVES * 64] * sb;
     }
   }
   const int lg = lane >> 4;
@@ -594,16 +649,17 @@ __device__ __forceinline__ void attend_block(BlockShared& sh, int item, int kvh,
 #define QUEUE_DONE 8
 #define QUEUE_INTS 16
 #if HD <= 128
-#define BLK_PER_CU 2
+#define BLK_PER_CU 2   // of the plain kind (GROUPS = 1); the kind with two groups fills a compute unit alone
 #else
 #define BLK_PER_CU 1
 #endif
-__global__ __launch_bounds__(64 * BLK_WAVES, BLK_PER_CU) void attn_mfma_block_kernel(
+template <int GROUPS>
+__global__ __launch_bounds__(64 * BLK_WAVES * GROUPS, GROUPS == 1 ? BLK_PER_CU : 1) void attn_mfma_block_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
     const int* __restrict__ bt, int table_width, const int* __restrict__ cu_q, const int* __restrict__ ctx_len,
     const int* __restrict__ blk_req, const int* __restrict__ blk_cb, int num_blocks, bf16_t* __restrict__ out, int nq,
     int nkv, int ps, int window, float scale, int* __restrict__ queue) {
-  __shared__ BlockShared sh;
+  __shared__ BlockShared<GROUPS> sh;
   const bool per_head = 8 % nkv == 0;
   const int queues = per_head ? nkv : 1;
   const int per_queue = per_head ? num_blocks : num_blocks * nkv;
@@ -759,23 +815,33 @@ static int check_common(int num_tiles, int nq, int nkv, int ps, int table_width)
 // workgroups a compute unit holds at a time.
 extern "C" int qvl_attn_mfma_block_tiles() { return BLK_WAVES * BLK_CT; }
 extern "C" int qvl_attn_mfma_block_per_cu() { return BLK_PER_CU; }
+extern "C" int qvl_attn_mfma_block_max_groups() { return BLK_MAX_GROUPS; }
 extern "C" int qvl_attn_mfma_queue_ints() { return QUEUE_INTS; }
 
 extern "C" int qvl_attn_mfma_block(const void* q, const void* kc, const void* vc, const void* bt, int table_width,
                                    const void* cu_q, const void* ctx_len, const void* blk_req, const void* blk_cb,
                                    int num_blocks, void* out, int nq, int nkv, int ps, int window, float scale,
-                                   void* queue, int max_workgroups, hipStream_t stream) {
-  // queue: qvl_attn_mfma_queue_ints() ints, zero before the first launch that uses them
+                                   void* queue, int max_workgroups, int groups, hipStream_t stream) {
+  // queue: qvl_attn_mfma_queue_ints() ints, zero before the first launch that uses them.
+  // groups: wave groups per workgroup, 1 .. qvl_attn_mfma_block_max_groups(); max_workgroups should
+  // be what the device holds at a time (qvl_attn_mfma_block_per_cu() per compute unit with one group, one with two).
   const int c = check_common(num_blocks, nq, nkv, ps, table_width);
   if (c >= 0) return c;
   if (!(scale > 0.f) || !queue || max_workgroups <= 0) return QVL_ERR_SHAPE;
+  if (groups < 1 || groups > BLK_MAX_GROUPS) return QVL_ERR_LIMIT;
   const long long total = (long long)num_blocks * nkv;
   if (total > 0x7fffffffLL) return QVL_ERR_LIMIT;
   const unsigned grid = (unsigned)(total < max_workgroups ? total : max_workgroups);
-  hipLaunchKernelGGL(attn_mfma_block_kernel, dim3(grid), dim3(64 * BLK_WAVES), 0, stream,
-                     (const bf16_t*)q, (const bf16_t*)kc, (const bf16_t*)vc, (const int*)bt, table_width,
-                     (const int*)cu_q, (const int*)ctx_len, (const int*)blk_req, (const int*)blk_cb, num_blocks,
-                     (bf16_t*)out, nq, nkv, ps, window, scale, (int*)queue);
+#define QVL_BLOCK_LAUNCH(G)                                                                                          \
+  hipLaunchKernelGGL(attn_mfma_block_kernel<G>, dim3(grid), dim3(64 * BLK_WAVES * G), 0, stream, (const bf16_t*)q,    \
+                     (const bf16_t*)kc, (const bf16_t*)vc, (const int*)bt, table_width, (const int*)cu_q,              \
+                     (const int*)ctx_len, (const int*)blk_req, (const int*)blk_cb, num_blocks, (bf16_t*)out, nq, nkv, \
+                     ps, window, scale, (int*)queue)
+  if (groups == 1) QVL_BLOCK_LAUNCH(1);
+#if BLK_MAX_GROUPS > 1
+  else QVL_BLOCK_LAUNCH(2);
+#endif
+#undef QVL_BLOCK_LAUNCH
   return qvl_launch_status();
 }
 

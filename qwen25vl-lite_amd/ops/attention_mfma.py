@@ -91,9 +91,20 @@ def _step_tiles(step, group: int, tile_ct: int, device, by_length: bool = False)
     return cache[key]
 
 
+def block_groups(walks: int, places: int, head_dim: int) -> int:
+    """Wave groups per workgroup for a step of ``walks`` (entry, head) pairs on a device that holds
+    ``places`` plain workgroups at a time.  Two groups (head sizes up to 128) halve a walk's time at
+    a tenth less throughput (measured at 2,048 to 8,192 tokens): they pay when all walks start at
+    once and the longest decides, not when places are taken several times over."""
+    most = int(_fn("attention_mfma", "qvl_attn_mfma_block_max_groups", [], {"HD": head_dim})())
+    return 2 if most >= 2 and walks <= places else 1
+
+
 def try_attention(q, k_cache, v_cache, block_table, step, num_q_heads: int, window: Optional[int],
-                  scale: float) -> Optional[torch.Tensor]:
-    """The attention through the matrix-core kernel, or None if it does not take this shape."""
+                  scale: float, force_groups: Optional[int] = None) -> Optional[torch.Tensor]:
+    """The attention through the matrix-core kernel, or None if it does not take this shape.
+    ``force_groups`` (tests): the workgroup kind of the kernel for prompt portions, else chosen by
+    :func:`block_groups`."""
     pages, nkv, ps, hd = k_cache.shape
     if not supports(hd, q.dtype) or ps % 16:
         return None
@@ -115,11 +126,12 @@ def try_attention(q, k_cache, v_cache, block_table, step, num_q_heads: int, wind
     if kind == "tile":
         fn = _fn("attention_mfma", "qvl_attn_mfma_block",
                  [_c_ptr] * 4 + [_c_int] + [_c_ptr] * 4 + [_c_int, _c_ptr] + [_c_int] * 4
-                 + [_c_float, _c_ptr, _c_int, _c_ptr], defines)
+                 + [_c_float, _c_ptr, _c_int, _c_int, _c_ptr], defines)
         queue, cus = _work_queue(q.device)
         per_cu = int(_fn("attention_mfma", "qvl_attn_mfma_block_per_cu", [], defines)())
-        _check(fn(*common, nq, nkv, ps, int(window or 0), float(scale), _ptr(queue), cus * per_cu, _stream()),
-               "paged_attention (matrix cores)")
+        groups = block_groups(num_tiles * nkv, cus * per_cu, hd) if force_groups is None else force_groups
+        _check(fn(*common, nq, nkv, ps, int(window or 0), float(scale), _ptr(queue),
+                  cus * (per_cu if groups == 1 else 1), groups, _stream()), "paged_attention (matrix cores)")
     else:
         scratch = None
         if nsplit > 1:

@@ -175,15 +175,20 @@ def test_paged_attention_generic(dtype, nq, nkv, hd, window):
     assert torch.allclose(out.float().cpu(), c["want"], **tol), (out.float().cpu() - c["want"]).abs().max()
 
 
-@pytest.mark.parametrize("split", ["tile", "coop", "coop_split"])
+@pytest.mark.parametrize("split", ["tile", "tile_two_groups", "coop", "coop_split"])
 @pytest.mark.parametrize("nq, nkv, hd, window", [s for s in ATTN_SHAPES if s[2] % 16 == 0])
 def test_paged_attention_matrix_cores(nq, nkv, hd, window, split, monkeypatch):
     """The matrix-core kernels on the same case: blocks that own several tiles and share the keys
-    through LDS, the waves of a block sharing one tile, and the keys further split among blocks."""
+    through LDS (one group of waves, or two that take the key blocks in turn and merge), the waves
+    of a block sharing one tile, and the keys further split among blocks."""
     from qwen25vl_lite_amd.ops import attention_mfma
     from qwen25vl_lite_amd.parts import StepContext
     c = _attention_case(torch.bfloat16, nq, nkv, hd, window)
-    plan = {"tile": ("tile", 1, 0), "coop": ("coop", 1, 0), "coop_split": ("coop", 6, 64)}[split]
+    plan = {"tile": ("tile", 1, 0), "tile_two_groups": ("tile", 1, 0), "coop": ("coop", 1, 0),
+            "coop_split": ("coop", 6, 64)}[split]
+    groups = {"tile": 1, "tile_two_groups": 2}.get(split)
+    if groups == 2 and hd > 128:
+        pytest.skip("two groups of waves are built for head sizes up to 128")
     monkeypatch.setattr(attention_mfma, "plan_splits", lambda t, n, m: plan)
     cu = [0]
     for ql in c["qlens"]:
@@ -194,7 +199,8 @@ def test_paged_attention_matrix_cores(nq, nkv, hd, window, split, monkeypatch):
                        ctx_len=torch.tensor(c["lens"], dtype=torch.int32).cuda(), req_slots=none, groups=[],
                        logit_rows=none, cu_q_host=cu, ctx_len_host=c["lens"], max_q_len=17, max_ctx_len=333,
                        dtype=torch.bfloat16)
-    out = attention_mfma.try_attention(c["q"], c["kc"], c["vc"], c["table"], step, nq, window, c["scale"])
+    out = attention_mfma.try_attention(c["q"], c["kc"], c["vc"], c["table"], step, nq, window, c["scale"],
+                                       force_groups=groups)
     assert out is not None
     err = (out.float().cpu() - c["want"]).abs().max()
     assert torch.allclose(out.float().cpu(), c["want"], atol=1.5e-2, rtol=2e-2), err
@@ -205,7 +211,7 @@ def test_paged_attention_long_portions(nq, nkv, hd, window):
     """Prompt portions long enough for several blocks of several waves per request, next to a
     short portion and a decoded token: the kernel that shares keys through LDS walks the union of
     its waves' ranges, with blocks that some of its waves skip."""
-    from qwen25vl_lite_amd.ops import attention_mfma
+    from qwen25vl_lite_amd.ops import attention_mfma, kernels
     from qwen25vl_lite_amd.parts import StepContext
     lens, qlens = (413, 150, 90), (380, 3, 1)
     c = _attention_case(torch.bfloat16, nq, nkv, hd, window, lens, qlens)
@@ -219,10 +225,16 @@ def test_paged_attention_long_portions(nq, nkv, hd, window):
                        logit_rows=none, cu_q_host=cu, ctx_len_host=list(lens), max_q_len=max(qlens),
                        max_ctx_len=max(lens), dtype=torch.bfloat16)
     import unittest.mock as mock
-    with mock.patch.object(attention_mfma, "plan_splits", lambda t, n, m: ("tile", 1, 0)):
-        out = attention_mfma.try_attention(c["q"], c["kc"], c["vc"], c["table"], step, nq, window, c["scale"])
-    err = (out.float().cpu() - c["want"]).abs().max()
-    assert torch.allclose(out.float().cpu(), c["want"], atol=1.5e-2, rtol=2e-2), err
+    for groups in (1, 2) if hd <= 128 else (1,):   # an odd and an even number of key blocks among the walks
+        with mock.patch.object(attention_mfma, "plan_splits", lambda t, n, m: ("tile", 1, 0)):
+            out = attention_mfma.try_attention(c["q"], c["kc"], c["vc"], c["table"], step, nq, window, c["scale"],
+                                               force_groups=groups)
+        err = (out.float().cpu() - c["want"]).abs().max()
+        assert torch.allclose(out.float().cpu(), c["want"], atol=1.5e-2, rtol=2e-2), (groups, err)
+    assert attention_mfma.block_groups(10, 512, hd) == (2 if hd <= 128 else 1)
+    assert attention_mfma.block_groups(513, 512, hd) == 1
+    with mock.patch.object(attention_mfma, "plan_splits", lambda t, n, m: ("tile", 1, 0)), pytest.raises(kernels.KernelError):
+        attention_mfma.try_attention(c["q"], c["kc"], c["vc"], c["table"], step, nq, window, c["scale"], force_groups=3)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
