@@ -142,22 +142,26 @@ struct Walk {
   __device__ __forceinline__ void compute(int kb, const bf16x8_t (*qb)[KS], const BlockRegs& rg, TileState* sts) const {
     const int key0 = kb << 5;
     const bool interior = key0 >= all_lo && key0 + 31 <= all_hi;
+    // the scores of all column tiles first: while the exponentials of one tile are taken, the
+    // matrix cores still work on the scores of the next
+    f32x4_t s[CT][2];
 #pragma unroll
-    for (int t = 0; t < CT; ++t) {
-      TileState& st = sts[t];
-      f32x4_t s[2];
+    for (int t = 0; t < CT; ++t)
 #pragma unroll
       for (int b = 0; b < 2; ++b) {
         f32x4_t a = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(rg.k[b][ks], qb[t][ks], a, 0, 0, 0);
-        s[b] = a;
+        s[t][b] = a;
       }
+#pragma unroll
+    for (int t = 0; t < CT; ++t) {
+      TileState& st = sts[t];
       // mask and online softmax; this lane holds keys key0 + 8*lg + j of column r.  A block that
       // lies wholly inside what every column of the wave sees needs no mask.
       float raw[8];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) raw[j] = (j < 4) ? s[0][j] : s[1][j - 4];
+      for (int j = 0; j < 8; ++j) raw[j] = (j < 4) ? s[t][0][j] : s[t][1][j - 4];
       if (!interior) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
