@@ -179,8 +179,11 @@ def main(argv=None) -> int:
                             max_model_len=max_ctx, enable_prefix_cache=True, dtype=dtype, device="cuda:0",
                             hip_graph=not args.no_graph, tune_library_products=not args.no_tune)
 
+        runner = ModelRunner(model, ecfg)        # one runner, as a server has: its decode graphs stay
+
         def serve():
-            runner = ModelRunner(model, ecfg)
+            if runner.cache.prefix_cache is not None:
+                runner.cache.prefix_cache.clear()  # every run starts without remembered prompts
             engine = LLMEngine(runner, ecfg)
             for tk, out in reqs:
                 engine.add_request(tk, SamplingParams(temperature=0.0, max_tokens=out, ignore_eos=True))
@@ -190,7 +193,7 @@ def main(argv=None) -> int:
             torch.cuda.synchronize()
             return time.perf_counter() - t0, outs, engine.stats()
 
-        serve()                                   # library tuning, kernel builds, first graph captures
+        serve()                                   # library tuning, kernel builds, graph captures
         sec, outs, stats = serve()
         generated = sum(len(o.output_token_ids) for o in outs)
         prompt_tokens = sum(len(tk) for tk, _ in reqs)

@@ -169,6 +169,18 @@ class RadixPrefixCache:
             evicted += self._drop(leaves[0])
         return evicted
 
+    def clear(self) -> int:
+        """Forget every entry that no running request uses (leaves first, so whole unused branches
+        go); their pages return to the pools unless a request still holds them.  Returns the number
+        of nodes dropped."""
+        dropped = 0
+        while True:
+            leaves = self._evictable_leaves()
+            if not leaves:
+                return dropped
+            for nid in leaves:
+                dropped += self._drop(nid)
+
     def held_pages(self, group: int) -> Dict[int, int]:
         out: Dict[int, int] = {}
         for nid, node in self.nodes.items():

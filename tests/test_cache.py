@@ -139,6 +139,24 @@ def test_prefix_eviction_returns_pages():
     assert len(pc) == 0 and pools[0].in_use() == 0
 
 
+def test_clearing_the_prefix_cache_keeps_what_is_in_use():
+    cm = _manager(windows=(None,), pages=8, page_size=4, seqs=3)
+    toks = list(range(100, 112))
+    cm.admit("a")
+    cm.reserve("a", 12)
+    cm.commit("a", 12)
+    assert cm.register_prefix("a", toks) == 3
+    cm.release("a")
+    cm.admit("b")
+    assert cm.adopt_prefix("b", toks[:8] + [1, 2]) == 8        # b uses the first two nodes
+    assert cm.prefix_cache.clear() == 1 and len(cm.prefix_cache) == 2
+    cm.check()
+    cm.release("b")
+    assert cm.prefix_cache.clear() == 2 and len(cm.prefix_cache) == 0
+    assert cm.pages_in_use() == [0]
+    cm.check()
+
+
 def test_pressure_evicts_unused_prefixes_but_not_used_ones():
     cm = _manager(windows=(None,), pages=4, page_size=4, seqs=3)
     toks = list(range(100, 112))
