@@ -2,7 +2,7 @@
 
     python bench.py --gpus 1 --steps K --warmup W
 
-The model has the layer sizes of BASELINE.json's configs[2] (the Qwen2.5-VL-7B text decoder)
+The model has the layer sizes of the Qwen2.5-VL-7B text decoder
 with random weights N(0, 0.02) in bfloat16; token ids are seeded uniform random integers.  A
 "step" is one decode step of the scheduler: every live request gets its next token through the
 engine's own path (batch building, the step function over the paged cache, sampling on the
@@ -27,7 +27,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 MFMA_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
 
 
-SIZES = {   # layer sizes of BASELINE.json's configs[3], [2] and [4]
+SIZES = {   # layer sizes of the Qwen2.5-VL 3B, 7B and 72B text decoders
     "3b": dict(hidden_size=2048, intermediate_size=11008, num_hidden_layers=36, num_attention_heads=16,
                num_key_value_heads=2, vocab_size=151936, tie_word_embeddings=True),
     "7b": dict(hidden_size=3584, intermediate_size=18944, num_hidden_layers=28, num_attention_heads=28,
@@ -38,7 +38,7 @@ SIZES = {   # layer sizes of BASELINE.json's configs[3], [2] and [4]
 
 
 def decoder_config(layers=None, size="7b"):
-    """configs[2] of BASELINE.json (or another of its sizes) as a config.json dictionary."""
+    """The 7B text decoder (or another of SIZES) as a config.json dictionary."""
     raw = {
         "architectures": ["Qwen2_5_VLForConditionalGeneration"], "model_type": "qwen2_5_vl",
         "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "sliding_window": 32768, "use_sliding_window": False,
@@ -84,7 +84,7 @@ def main(argv=None) -> int:
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and the prefill")
     ap.add_argument("--prefill-only", action="store_true", help="only the 2,048-token prefill (for profiles)")
     ap.add_argument("--serving", action="store_true",
-                    help="instead: continuous batching of 64 requests (BASELINE.json configs[3]'s workload: prompts "
+                    help="instead: continuous batching of 64 requests (prompts "
                          "of 64 to 2048 tokens, 32 to 512 generated, a quarter sharing a 1024-token prefix)")
     ap.add_argument("--no-graph", action="store_true", help="do not replay decode steps from a HIP graph")
     ap.add_argument("--no-tune", action="store_true", help="do not let TunableOp choose the library's kernels")

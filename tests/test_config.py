@@ -9,7 +9,7 @@ from conftest import TINY_A, TINY_B, TINY_C
 from qwen25vl_lite_amd import ConfigError, Qwen25VLConfig, build_model, known_architectures, register_architecture
 from qwen25vl_lite_amd.config import EngineConfig, resolve_architecture
 
-SEVEN_B = {  # sizes of BASELINE configs[2]
+SEVEN_B = {  # sizes of the Qwen2.5-VL-7B text decoder
     "architectures": ["Qwen2_5_VLForConditionalGeneration"], "tie_word_embeddings": False,
     "hidden_size": 3584, "intermediate_size": 18944, "num_hidden_layers": 28, "num_attention_heads": 28,
     "num_key_value_heads": 4, "vocab_size": 152064, "rope_theta": 1e6, "rms_norm_eps": 1e-6,
