@@ -451,7 +451,12 @@ struct BlockLoader {
     for (int i = 0; i < WAVE_LOADS; ++i) {
       const int t = load_index(i);
       const bool second = (halves >> i) & 1u;
-      const bf16_t* base = t < K_LOADS ? (second ? kh[1] : kh[0]) : (second ? vh[1] : vh[0]);
+      // keys or values is the same for the whole wave: chosen in scalar registers, before the lanes
+      // choose their half
+      const bool keys = t < K_LOADS;
+      const bf16_t* first_half = keys ? kh[0] : vh[0];
+      const bf16_t* second_half = keys ? kh[1] : vh[1];
+      const bf16_t* base = second ? second_half : first_half;
       load16_to_lds(base + fixed[i], __builtin_amdgcn_readfirstlane(stage + 1024u * t));
     }
   }
