@@ -35,7 +35,10 @@ class EngineConfig:
     ``max_num_batched_tokens`` tokens, decoded tokens included; ``max_model_len`` bounds a
     request's prompt plus output.  ``preemption`` is what happens when pages run out:
     only ``"recompute"`` is built (the victim gives its pages back and is prefilled again,
-    prompt and tokens generated so far).  ``hip_graph`` replays decode steps from captured HIP graphs.
+    prompt and tokens generated so far).  ``hip_graph`` replays decode steps from captured HIP graphs;
+    with ``decode_lookahead`` the scheduler then queues the decode step after the running one before
+    the host has seen the running one's tokens (the ids go from the sampler to the next step on the
+    device), so that the GPU does not wait for the host between steps.
     ``tune_library_products`` lets PyTorch's TunableOp choose the library kernel of each product shape
     (seconds per new shape, once): for runs with few distinct step sizes.
     """
@@ -51,6 +54,7 @@ class EngineConfig:
     device: str = "cuda:0"
     dtype: torch.dtype = torch.float32
     hip_graph: bool = False
+    decode_lookahead: bool = True
     tune_library_products: bool = False
 
     def __post_init__(self) -> None:

@@ -20,7 +20,7 @@ the attention kernel splits a request's keys over; the true lengths travel in th
 
 from __future__ import annotations
 
-from typing import Dict, List, Sequence, Tuple
+from typing import Dict, List, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
@@ -144,11 +144,15 @@ class _Graph:
         for i in range(n, b):
             self.row_req[i] = None
 
-    def run(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def run(self, entries: Sequence[StepEntry], device_tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
         runner = self.runner
         self.fill(entries)
         self.dev.copy_(self.host, non_blocking=True)
         self.copied.record()
+        if device_tokens is not None:
+            # the entries' token ids are still on the device (sampled by the step before, whose ids
+            # the host has not seen): they go into the step's input without a detour
+            self.step.token_ids[:len(entries)].copy_(device_tokens)
         if self.graph is None:
             # twice eagerly (libraries pick kernels and workspaces, per-step tile lists are made),
             # then once more under capture; a decode step only writes the step's own cache slots
@@ -178,7 +182,7 @@ class DecodeGraphs:
     def takes(entries: Sequence[StepEntry]) -> bool:
         return all(len(e.tokens) == 1 and e.positions is None and list(e.want) == [0] for e in entries)
 
-    def run(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def run(self, entries: Sequence[StepEntry], device_tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
         ctx = max(e.start for e in entries) + 1
         key = (_batch_bucket(len(entries), self.runner.ecfg.max_num_seqs), _bucket(ctx))
         g = self.graphs.get(key)
@@ -186,4 +190,4 @@ class DecodeGraphs:
             if len(self.graphs) >= self.max_graphs:
                 self.graphs.pop(next(iter(self.graphs)))
             g = self.graphs[key] = _Graph(self.runner, *key)
-        return g.run(entries)
+        return g.run(entries, device_tokens)

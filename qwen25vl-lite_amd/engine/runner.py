@@ -88,10 +88,14 @@ class ModelRunner:
 
     # ------------------------------------------------------------------ the step
     @torch.no_grad()
-    def execute(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def execute(self, entries: Sequence[StepEntry], device_tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Run one step.  Pages for the new tokens are reserved here if the caller has not done
         so (:class:`~qwen25vl_lite_amd.cache.OutOfPages` if they cannot be).  Returns float32 logits
-        ``[wanted, vocab]`` in the order of the entries and of each entry's ``want``."""
+        ``[wanted, vocab]`` in the order of the entries and of each entry's ``want``.
+
+        ``device_tokens`` (int32 ``[len(entries)]`` on the device): the entries' single tokens, for
+        a step that :meth:`decodes_from_graph` and is queued before the host has seen the ids the
+        step before it sampled; the entries' own token ids are placeholders then."""
         for e in entries:
             self.cache.reserve(e.req_id, e.start + len(e.tokens))
         self._clear_state(entries)
@@ -102,7 +106,9 @@ class ModelRunner:
                         raise ValueError(f"request {e.req_id!r}: token id outside [0, {self.vocab_size})")
                     if self.cache.num_tokens(e.req_id) != e.start:
                         raise ValueError(f"request {e.req_id!r}: the step does not continue where the cache ends")
-                logits = self.graphs.run(entries)
+                logits = self.graphs.run(entries, device_tokens)
+            elif device_tokens is not None:
+                raise ValueError("token ids on the device are taken by decode steps that run from a graph only")
             else:
                 step = build_step(entries, self.cache, self.position_rows, self.dtype, self.device, self.vocab_size)
                 logits = self.model.forward(step, self.slots)
@@ -110,6 +116,18 @@ class ModelRunner:
             self.cache.commit(e.req_id, e.start + len(e.tokens))
         self.steps += 1
         return logits
+
+    def decodes_from_graph(self, entries: Sequence[StepEntry]) -> bool:
+        """Whether :meth:`execute` would replay these entries from a decode graph."""
+        return self.graphs is not None and self.graphs.takes(entries)
+
+    def sample_begin(self, logits: torch.Tensor, params: Sequence, prev_ids: Sequence[Sequence[int]],
+                     steps: Sequence[int]):
+        """Queue the sampling; the returned object has ``device_ids`` and ``result()`` (see
+        :class:`~qwen25vl_lite_amd.sampling.sampler.PendingSample`)."""
+        from ..sampling.sampler import sample_rows_begin
+        with torch.cuda.device(self.device):
+            return sample_rows_begin(logits, params, prev_ids, steps)
 
     def sample(self, logits: torch.Tensor, params: Sequence, prev_ids: Sequence[Sequence[int]],
                steps: Sequence[int]) -> List[int]:

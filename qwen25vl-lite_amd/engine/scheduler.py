@@ -110,6 +110,7 @@ class LLMEngine:
         self.finished: List[RequestOutput] = []
         self.stats_ = EngineStats()
         self._next_id = 0
+        self._ahead: Optional[Tuple[List[Tuple[Sequence_, int]], List[StepEntry], object]] = None
         self.position_rows = getattr(runner, "position_rows", 3)
 
     # ------------------------------------------------------------------ requests
@@ -273,14 +274,25 @@ class LLMEngine:
     def step(self) -> List[RequestOutput]:
         """One scheduling iteration; returns the requests that finished in it."""
         done: List[RequestOutput] = []
-        plan = self._schedule()
-        self.stats_.steps += 1
-        if not plan:
-            return done
-        entries = [self._entry(seq, n) for seq, n in plan]
-        logits = self.runner.execute(entries)
+        ahead, self._ahead = self._ahead, None
+        if ahead is not None and not any(seq.status == "running" for seq, _ in ahead[0]):
+            ahead = None                       # everyone in the step queued ahead has finished since
+        if ahead is not None:
+            plan, entries, logits = ahead      # queued by the step before (see _queue_ahead)
+            self.stats_.steps += 1
+        else:
+            plan = self._schedule()
+            self.stats_.steps += 1
+            if not plan:
+                return done
+            entries = [self._entry(seq, n) for seq, n in plan]
+            logits = self.runner.execute(entries)
         sampled: List[Sequence_] = []
-        for (seq, n), entry in zip(plan, entries):
+        rows: List[int] = []
+        for row, ((seq, n), entry) in enumerate(zip(plan, entries)):
+            if seq.status != "running":
+                continue   # it finished after this step was queued ahead: its row is computed for nothing
+            rows.append(row)
             was_prompt = seq.num_computed_tokens < len(seq.prompt_token_ids)
             seq.num_computed_tokens += n
             self.stats_.batched_tokens += n
@@ -293,13 +305,60 @@ class LLMEngine:
             if entry.want:
                 sampled.append(seq)
         if sampled:
-            tokens = self.runner.sample(logits, [s.params for s in sampled],
-                                        [s.output_token_ids for s in sampled],
-                                        [len(s.output_token_ids) for s in sampled])
+            args = ([s.params for s in sampled], [s.output_token_ids for s in sampled],
+                    [len(s.output_token_ids) for s in sampled])
+            if ahead is not None and len(rows) < len(plan):
+                logits = logits[rows]          # every entry of a step queued ahead wants one row
+            if self._may_look_ahead(plan, sampled):
+                pending = self.runner.sample_begin(logits, *args)
+                self._queue_ahead(sampled, pending)
+                tokens = pending.result()
+            else:
+                tokens = self.runner.sample(logits, *args)
             for seq, token in zip(sampled, tokens):
                 self._accept(seq, int(token), done)
         self.finished.extend(done)
         return done
+
+    # ------------------------------------------------------------------ looking one step ahead
+    def _may_look_ahead(self, plan: List[Tuple[Sequence_, int]], sampled: List[Sequence_]) -> bool:
+        """Whether the step after this one can be queued before this one's tokens are known: it is a
+        decode step of exactly the requests sampled now (nobody waits for admission, nobody is left
+        out or still in its prompt), and no request's sampling reads the tokens it generated."""
+        if not (self.ecfg.hip_graph and self.ecfg.decode_lookahead and hasattr(self.runner, "sample_begin")):
+            return False
+        if self.waiting or len(sampled) != len(self.running):
+            return False
+        return all(s.params.repetition_penalty == 1.0 and s.params.presence_penalty == 0.0
+                   and s.params.frequency_penalty == 0.0 for s in sampled)
+
+    def _queue_ahead(self, sampled: List[Sequence_], pending) -> None:
+        """Queue the next decode step on the GPU.  Its token ids are the ones being sampled, taken
+        on the device.  Requests that are known to end with this token (length) are left out; one
+        that ends on a stop token is found out only afterwards: its row of the queued step is then
+        computed for nothing and ignored, and what it writes lands in pages that are free again,
+        before any later step's own writes to them.  Nothing else differs from scheduling the
+        step afterwards: rows do not depend on each other."""
+        keep = [i for i, s in enumerate(sampled)
+                if len(s.output_token_ids) + 1 < s.params.max_tokens and s.num_tokens + 1 < self.ecfg.max_model_len]
+        if not keep or len(keep) > self.ecfg.max_num_batched_tokens:
+            return
+        cache = self.runner.cache
+        seqs = [sampled[i] for i in keep]
+        entries = [StepEntry(req_id=s.seq_id, tokens=[0], start=s.num_computed_tokens, want=[0], positions=None,
+                             rope_delta=s.rope_delta) for s in seqs]
+        if not self.runner.decodes_from_graph(entries):
+            return
+        try:
+            for s in seqs:
+                cache.reserve(s.seq_id, s.num_computed_tokens + 1)
+        except OutOfPages:
+            return      # the scheduler decides who gives way, with the tokens known
+        ids = pending.device_ids
+        if len(keep) < len(sampled):
+            ids = ids[keep]
+        logits = self.runner.execute(entries, device_tokens=ids)
+        self._ahead = ([(s, 1) for s in seqs], entries, logits)
 
     def _accept(self, seq: Sequence_, token: int, done: List[RequestOutput]) -> None:
         """Append a sampled token and finish the request if it must (reference engine.py:831-872)."""

@@ -17,7 +17,7 @@ import torch
 from ..ops.kernels import KernelError, _check, _fn, _stream
 from .params import SamplingParams
 
-__all__ = ["sample_rows", "uniform_for"]
+__all__ = ["sample_rows", "sample_rows_begin", "PendingSample", "uniform_for"]
 
 _ROW = np.dtype([("temperature", "<f4"), ("top_p", "<f4"), ("min_p", "<f4"), ("u", "<f4"),
                  ("repetition", "<f4"), ("presence", "<f4"), ("frequency", "<f4"), ("top_k", "<i4"),
@@ -35,6 +35,60 @@ def uniform_for(params: SamplingParams, step: int) -> float:
     return float(torch.rand(1, generator=gen).item())
 
 
+class _Staging:
+    """Pinned host buffers that take turns carrying the sampler's per-row settings to the device:
+    a copy from pinned memory does not make the host wait for the work queued before it."""
+
+    _rings = {}
+
+    @classmethod
+    def to_device(cls, packed: np.ndarray, device: torch.device) -> torch.Tensor:
+        key = device.index or 0
+        ring = cls._rings.setdefault(key, {"turn": -1, "slots": [None] * 4})
+        turn = ring["turn"] = (ring["turn"] + 1) % len(ring["slots"])
+        slot = ring["slots"][turn]
+        if slot is None or slot[0].numel() < packed.size:
+            slot = ring["slots"][turn] = (torch.empty(max(1024, 2 * packed.size), dtype=torch.int32, pin_memory=True),
+                                         torch.cuda.Event())
+        else:
+            slot[1].synchronize()       # the copy that last read this buffer is done
+        host, copied = slot
+        host.numpy()[:packed.size] = packed
+        buf = torch.empty(packed.size, dtype=torch.int32, device=device)
+        buf.copy_(host[:packed.size], non_blocking=True)
+        copied.record()
+        return buf
+
+
+class PendingSample:
+    """Sampled ids that are on their way: ``device_ids`` (int32 ``[M]``, valid for kernels queued
+    after the sampler on the same stream) and a copy to pinned host memory whose end an event
+    marks.  :meth:`result` waits for that copy only, not for work queued after it."""
+
+    _pinned = {}     # device index -> ring of pinned int32 buffers, so that two samples can be pending
+    _turn = {}
+
+    def __init__(self, device_ids: torch.Tensor):
+        m = device_ids.numel()
+        key = device_ids.device.index or 0
+        ring = self._pinned.setdefault(key, [None] * 4)
+        turn = self._turn[key] = (self._turn.get(key, -1) + 1) % len(ring)
+        if ring[turn] is None or ring[turn].numel() < m:
+            ring[turn] = torch.empty(max(256, m), dtype=torch.int32, pin_memory=True)
+        self.device_ids = device_ids
+        self._host = ring[turn][:m]
+        self._host.copy_(device_ids, non_blocking=True)
+        self._event = torch.cuda.Event()
+        self._event.record()
+        self._ids: Optional[List[int]] = None
+
+    def result(self) -> List[int]:
+        if self._ids is None:
+            self._event.synchronize()
+            self._ids = self._host.tolist()
+        return self._ids
+
+
 def sample_rows(logits: torch.Tensor, params: Sequence[SamplingParams], prev_ids: Sequence[Sequence[int]],
                 steps: Sequence[int], uniforms: Optional[Sequence[float]] = None) -> List[int]:
     """Sample a token for each row of float32 ``logits [M, vocab]`` on the GPU.
@@ -42,6 +96,14 @@ def sample_rows(logits: torch.Tensor, params: Sequence[SamplingParams], prev_ids
     ``prev_ids[m]`` are the tokens request ``m`` has generated so far (for the penalties) and
     ``steps[m]`` their number (for the seed rule).  ``uniforms`` overrides the random numbers.
     """
+    pending = sample_rows_begin(logits, params, prev_ids, steps, uniforms)
+    return pending.result() if pending is not None else []
+
+
+def sample_rows_begin(logits: torch.Tensor, params: Sequence[SamplingParams], prev_ids: Sequence[Sequence[int]],
+                      steps: Sequence[int], uniforms: Optional[Sequence[float]] = None) -> Optional[PendingSample]:
+    """Queue the sampling of :func:`sample_rows` and the copy of its ids to the host; nothing is
+    waited for.  None for no rows."""
     if not logits.is_cuda:
         raise KernelError("sampling has no CPU path: logits must be on the GPU")
     if logits.dtype != torch.float32 or logits.dim() != 2 or not logits.is_contiguous():
@@ -50,7 +112,7 @@ def sample_rows(logits: torch.Tensor, params: Sequence[SamplingParams], prev_ids
     if not (len(params) == len(prev_ids) == len(steps) == m):
         raise ValueError("one SamplingParams, token list and step per logits row is needed")
     if m == 0:
-        return []
+        return None
     rows = np.zeros(m, _ROW)
     flat: List[int] = []
     first = params[0]
@@ -75,7 +137,7 @@ def sample_rows(logits: torch.Tensor, params: Sequence[SamplingParams], prev_ids
     dev = logits.device
     with torch.cuda.device(dev):
         packed = np.concatenate([rows.view(np.int32), np.asarray(flat or [0], np.int32)])
-        buf = torch.from_numpy(packed).to(dev)
+        buf = _Staging.to_device(packed, dev)
         n_row_words = rows.view(np.int32).size
         need_scores = any(p.temperature > 0 or len(flat) for p in params)
         scores = torch.empty_like(logits) if need_scores else logits
@@ -89,4 +151,4 @@ def sample_rows(logits: torch.Tensor, params: Sequence[SamplingParams], prev_ids
         _check(fn(logits.data_ptr(), scores.data_ptr(), buf.data_ptr(), buf[n_row_words:].data_ptr(),
                   parts.data_ptr() if parts is not None else None, out.data_ptr(), m, vocab, _stream()),
                "sample_rows")
-        return out.cpu().tolist()
+        return PendingSample(out)

@@ -123,6 +123,57 @@ def test_decode_graphs_with_padding_rows(model_dirs, name, dtype):
     assert llm.runner.cache.pages_in_use() == [0] * len(llm.runner.cache.groups)
 
 
+@pytest.mark.parametrize("name, dtype", [("B_sharp", "float32"), ("C", "bfloat16")])
+def test_decode_step_queued_ahead_changes_nothing(model_dirs, name, dtype):
+    """With decode graphs the scheduler queues the next decode step before it has seen the running
+    step's tokens.  Requests that stop on a token (found out one step late), on their length
+    (known beforehand), that sample with a seed, that arrive while others decode, and one whose
+    penalties switch the lookahead off while it runs: tokens and finish reasons are those of the
+    engine that schedules every step afterwards (requests that arrive while a step is queued are
+    admitted one step later), and every page comes back."""
+    from qwen25vl_lite_amd import LLM, SamplingParams
+
+    d = model_dirs[name]
+    vocab = {"B": 509, "C": 300}[name[0]]
+    prompts = [random_tokens(n, vocab, 900 + n) for n in (12, 5, 30, 9, 17, 3)]
+    def run(lookahead, stops):
+        llm = LLM(d, dtype=dtype, num_blocks=64, block_size=16, max_num_seqs=6, max_num_batched_tokens=64,
+                  enable_prefix_cache=False, hip_graph=True, decode_lookahead=lookahead)
+        runner, engine = llm.runner, llm.engine
+        params = [SamplingParams(temperature=0.0, max_tokens=40, ignore_eos=True, stop_token_ids=stops[0]),
+                  SamplingParams(temperature=0.8, top_k=20, seed=5, max_tokens=23, ignore_eos=True),
+                  SamplingParams(temperature=0.0, max_tokens=31, ignore_eos=True, stop_token_ids=stops[2]),
+                  SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True),
+                  SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True, repetition_penalty=1.3),
+                  SamplingParams(temperature=1.1, top_p=0.9, seed=11, max_tokens=19, ignore_eos=True)]
+        for p, sp in zip(prompts[:3], params[:3]):
+            engine.add_request(p, sp)
+        steps = queued = 0
+        while engine.has_work():
+            engine.step()
+            steps += 1
+            queued += engine._ahead is not None
+            if steps == 6:            # three more arrive while the first three decode
+                for p, sp in zip(prompts[3:], params[3:]):
+                    engine.add_request(p, sp)
+        outs = sorted(engine.finished, key=lambda o: o.seq_id)
+        assert runner.cache.pages_in_use() == [0] * len(runner.cache.groups)
+        runner.cache.check()
+        return [(o.output_token_ids, o.finish_reason) for o in outs], steps, queued
+
+    free, _, _ = run(False, [(), (), ()])
+    # stop tokens that the requests really produce, in the middle of their outputs
+    stops = [(free[0][0][14],), (), (free[2][0][6],)]
+    plain, plain_steps, none_queued = run(False, stops)
+    ahead, ahead_steps, queued = run(True, stops)
+    assert none_queued == 0 and queued > 10, queued
+    assert plain[0][1] == "stop" and plain[2][1] == "stop" and len(plain[0][0]) <= 15
+    assert ahead == plain
+    assert ahead_steps in (plain_steps, plain_steps + 1)   # the arrivals wait for the step that was queued already
+    if dtype == "float32":
+        assert plain[3][0] == _plain_greedy(d, prompts[3], 8)
+
+
 @pytest.mark.parametrize("name, hip_graph", [("C_sharp", False), ("B_sharp", True)])
 def test_twenty_odd_requests_decode_together(model_dirs, name, hip_graph):
     """Between 17 and 32 decoded tokens a step the bfloat16 products run with two column tiles of
