@@ -13,9 +13,10 @@
 // Up to 16 rows of X are one column tile of the matrix instruction; 17 to 32 rows are two (MT = 2):
 // every W fragment that is loaded is multiplied with both.
 // If K fits one pass (K <= 4096) the X operand stays in registers (the second column tile, if
-// there is one, in LDS, which takes K <= 32 * XHI_STEPS) for all of the block's tiles and
-// the W loads of the next tile are issued before the current tile's sums are merged; a longer K is
-// walked in passes of 4096.
+// there is one, in LDS, which takes K <= 32 * XHI_STEPS) for all of the block's tiles; W comes
+// through three half-tile buffers that go round, so that the next tile and a half are on their way
+// while a tile is multiplied and its sums are merged.  A longer K is walked in passes of 4096 that
+// take their turns in the same rotation (X is then read again for every pass).
 //
 // What is folded in:
 //   prologue  PRO_NORM      X = rmsnorm(H) * w, from the float32 residual H (statistics in float32,
