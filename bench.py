@@ -87,6 +87,8 @@ def main(argv=None) -> int:
                     help="instead: continuous batching of 64 requests (prompts "
                          "of 64 to 2048 tokens, 32 to 512 generated, a quarter sharing a 1024-token prefix)")
     ap.add_argument("--no-graph", action="store_true", help="do not replay decode steps from a HIP graph")
+    ap.add_argument("--no-lookahead", action="store_true",
+                    help="do not queue the next decode step before the running one's tokens are known")
     ap.add_argument("--no-tune", action="store_true", help="do not let TunableOp choose the library's kernels")
     args = ap.parse_args(argv)
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -114,7 +116,7 @@ def main(argv=None) -> int:
         ecfg = EngineConfig(num_blocks=max_seqs * ((tokens_per_seq + page - 1) // page + 1), block_size=page,
                             max_num_seqs=max_seqs, max_num_batched_tokens=budget, max_model_len=max_ctx,
                             enable_prefix_cache=False, dtype=dtype, device="cuda:0", hip_graph=not args.no_graph,
-                            tune_library_products=not args.no_tune)
+                            decode_lookahead=not args.no_lookahead, tune_library_products=not args.no_tune)
         runner = ModelRunner(model, ecfg)
         return LLMEngine(runner, ecfg), runner
 
@@ -144,6 +146,7 @@ def main(argv=None) -> int:
         tokens = engine.stats_.decode_tokens - before
         assert tokens == batch * steps, (tokens, batch, steps)
         ctx_mid = args.prompt_tokens + warmup + steps // 2
+        runner.close()                         # the captured graphs go now, not when a collector runs
         del engine, runner
         torch.cuda.empty_cache()
         return tokens / dt, dt / steps * 1e3, ctx_mid
@@ -161,6 +164,7 @@ def main(argv=None) -> int:
             assert len(done) == 1
             if i:
                 times.append(time.perf_counter() - t0)
+        runner.close()                         # the captured graphs go now, not when a collector runs
         del engine, runner
         torch.cuda.empty_cache()
         return min(times)
@@ -177,7 +181,8 @@ def main(argv=None) -> int:
         need_pages = sum((len(tk) + out + page - 1) // page + 1 for tk, out in reqs)
         ecfg = EngineConfig(num_blocks=need_pages, block_size=page, max_num_seqs=64, max_num_batched_tokens=4096,
                             max_model_len=max_ctx, enable_prefix_cache=True, dtype=dtype, device="cuda:0",
-                            hip_graph=not args.no_graph, tune_library_products=not args.no_tune)
+                            hip_graph=not args.no_graph, decode_lookahead=not args.no_lookahead,
+                            tune_library_products=not args.no_tune)
 
         runner = ModelRunner(model, ecfg)        # one runner, as a server has: its decode graphs stay
 
@@ -226,7 +231,8 @@ def main(argv=None) -> int:
             "kv_heads": t.num_key_value_heads, "head_dim": t.head_dim, "intermediate_size": t.intermediate_size,
             "vocab_size": t.vocab_size, "global_batch": args.batch, "seq_len": args.prompt_tokens,
             "context_mid": ctx_mid, "max_context": max_ctx, "page_size": page, "parallelism": "single GPU",
-            "hip_graph": not args.no_graph, "tuned_library_products": not args.no_tune,
+            "hip_graph": not args.no_graph, "decode_lookahead": not (args.no_graph or args.no_lookahead),
+            "tuned_library_products": not args.no_tune,
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},

@@ -32,7 +32,7 @@ def _llm(args):
         num_blocks=args.num_blocks, block_size=args.block_size, max_num_seqs=args.max_num_seqs,
         max_num_batched_tokens=args.max_num_batched_tokens, max_model_len=args.max_model_len,
         enable_prefix_cache=not args.no_prefix_cache, enable_chunked_prefill=not args.no_chunked_prefill,
-        preemption=args.preemption, hip_graph=args.cuda_graph, decode_lookahead=not args.no_decode_lookahead)
+        preemption=args.preemption, hip_graph=args.cuda_graph, decode_lookahead=args.decode_lookahead)
     t0 = time.time()
     if args.random_weights is not None:
         llm = LLM(Qwen25VLConfig.from_pretrained(args.model), args.dtype, random_seed=args.random_weights,
@@ -133,9 +133,9 @@ def build_parser() -> argparse.ArgumentParser:
         p.add_argument("--no-prefix-cache", action="store_true")
         p.add_argument("--no-chunked-prefill", action="store_true")
         p.add_argument("--preemption", default="recompute", choices=["recompute"])
-        p.add_argument("--no-decode-lookahead", action="store_true",
-                       help="with --cuda-graph: do not queue the next decode step before the running one's "
-                            "tokens have reached the host")
+        p.add_argument("--decode-lookahead", action="store_true",
+                       help="with --cuda-graph: queue the next decode step before the running one's tokens "
+                            "have reached the host")
         p.add_argument("--cuda-graph", action="store_true",
                        help="replay decode steps from a captured graph (a HIP graph here; the option keeps "
                             "the reference's name): a decode step is launch-bound, this removes the host's "

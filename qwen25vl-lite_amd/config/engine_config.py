@@ -36,7 +36,7 @@ class EngineConfig:
     request's prompt plus output.  ``preemption`` is what happens when pages run out:
     only ``"recompute"`` is built (the victim gives its pages back and is prefilled again,
     prompt and tokens generated so far).  ``hip_graph`` replays decode steps from captured HIP graphs;
-    with ``decode_lookahead`` the scheduler then queues the decode step after the running one before
+    with ``decode_lookahead`` (off unless asked for) the scheduler then queues the decode step after the running one before
     the host has seen the running one's tokens (the ids go from the sampler to the next step on the
     device), so that the GPU does not wait for the host between steps.
     ``tune_library_products`` lets PyTorch's TunableOp choose the library kernel of each product shape
@@ -54,7 +54,7 @@ class EngineConfig:
     device: str = "cuda:0"
     dtype: torch.dtype = torch.float32
     hip_graph: bool = False
-    decode_lookahead: bool = True
+    decode_lookahead: bool = False
     tune_library_products: bool = False
 
     def __post_init__(self) -> None:

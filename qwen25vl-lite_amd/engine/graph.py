@@ -16,10 +16,20 @@ row; their logits are computed and dropped.
 
 The context bucket (the next power of two above the longest context) only fixes how many waves
 the attention kernel splits a request's keys over; the true lengths travel in the buffer.
+
+Lifetime.  A captured graph must never be destroyed while another capture is under way: its
+destructor synchronizes the device, which a capture refuses, and an error thrown from a
+destructor ends the process.  So nothing here refers back to the runner that owns it (a graph
+holds the model, the cache and the slots, none of which know the runner): an engine that is
+dropped frees its graphs at once, by reference count, not whenever the cycle collector next
+runs.  A capture starts with a collection (garbage of the caller's own may hold graphs) and
+keeps the collector off until it ends, and :meth:`DecodeGraphs.close` drops every graph after a
+device synchronization for callers that want it done at a place of their choosing.
 """
 
 from __future__ import annotations
 
+import gc
 from typing import Dict, List, Optional, Sequence, Tuple
 
 import numpy as np
@@ -51,13 +61,13 @@ def _bucket(n: int, floor: int = 256) -> int:
 class _Graph:
     """One captured step shape: its buffers, its StepContext of fixed views, its graph."""
 
-    def __init__(self, runner, batch: int, ctx_bucket: int):
-        self.runner = runner
+    def __init__(self, parts: "_RunnerParts", batch: int, ctx_bucket: int):
+        self.parts = parts
         self.batch = batch
-        cache = runner.cache
+        cache = parts.cache
         self.ngroups = len(cache.groups)
-        self.rows = runner.model.spec.position_rows
-        self.width = runner.ecfg.max_blocks_per_seq
+        self.rows = parts.model.spec.position_rows
+        self.width = parts.max_blocks_per_seq
         self.ps = cache.page_size
         b, w = batch, self.width
         sizes = [("token_ids", b), ("positions", self.rows * b), ("token_req", b), ("token_seqpos", b),
@@ -71,21 +81,10 @@ class _Graph:
             total += (n + 3) // 4 * 4
         self.host = torch.zeros(total, dtype=torch.int32, pin_memory=True)
         self.hv = self.host.numpy()
-        self.dev = torch.zeros(total, dtype=torch.int32, device=runner.device)
+        self.dev = torch.zeros(total, dtype=torch.int32, device=parts.device)
         self.copied = torch.cuda.Event()
         self.copied.record()
-
-        def h(name, shape=None):
-            o, n = self.offsets[name]
-            v = self.hv[o:o + n]
-            return v if shape is None else v.reshape(shape)
-
-        def d(name, shape=None):
-            o, n = self.offsets[name]
-            v = self.dev[o:o + n]
-            return v if shape is None else v.view(shape)
-
-        self.h = h
+        h, d = self.h, self._d
         h("token_req")[:] = np.arange(b)
         h("cu_q")[:] = np.arange(b + 1)
         h("logit_rows")[:] = np.arange(b)
@@ -100,12 +99,23 @@ class _Graph:
             req_slots=d("req_slots"),
             groups=[GroupStep(d(f"slots{g}"), d(f"table{g}", (b, w)), self.ps) for g in range(self.ngroups)],
             logit_rows=d("logit_rows"), cu_q_host=list(range(b + 1)), ctx_len_host=[ctx_bucket] * b,
-            req_slots_host=[0] * b, max_q_len=1, max_ctx_len=ctx_bucket, dtype=runner.dtype)
+            req_slots_host=[0] * b, max_q_len=1, max_ctx_len=ctx_bucket, dtype=parts.dtype)
         self.graph = None
         self.logits = None
 
+    def h(self, name, shape=None):
+        """The named array of the pinned host buffer."""
+        o, n = self.offsets[name]
+        v = self.hv[o:o + n]
+        return v if shape is None else v.reshape(shape)
+
+    def _d(self, name, shape=None):
+        o, n = self.offsets[name]
+        v = self.dev[o:o + n]
+        return v if shape is None else v.view(shape)
+
     def fill(self, entries: Sequence[StepEntry]) -> None:
-        cache, ps, h = self.runner.cache, self.ps, self.h
+        cache, ps, h = self.parts.cache, self.ps, self.h
         n, b = len(entries), self.batch
         self.copied.synchronize()          # the previous transfer has read the pinned buffer
         starts = np.zeros(b, np.int32)     # rows from n on are padding: position 0, one key, no slot
@@ -120,7 +130,7 @@ class _Graph:
         h("ctx_len")[:] = starts + 1
         slots_of = h("req_slots")
         slots_of[:n] = np.fromiter((cache.slot_of(e.req_id) for e in entries), np.int32, n)
-        slots_of[n:] = self.runner.pad_state_slot
+        slots_of[n:] = self.parts.pad_state_slot
         for g in range(self.ngroups):
             table_np, lens, slots = self.tables[g], self.row_len[g], h(f"slots{g}")
             for i, e in enumerate(entries):
@@ -145,7 +155,7 @@ class _Graph:
             self.row_req[i] = None
 
     def run(self, entries: Sequence[StepEntry], device_tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
-        runner = self.runner
+        parts = self.parts
         self.fill(entries)
         self.dev.copy_(self.host, non_blocking=True)
         self.copied.record()
@@ -159,24 +169,61 @@ class _Graph:
             # and the logits, so running it again with the same inputs changes nothing
             for _ in range(2):
                 self.step.per_pass.clear()
-                runner.model.forward(self.step, runner.slots)
+                parts.model.forward(self.step, parts.slots)
             torch.cuda.synchronize()
             self.step.per_pass.clear()    # what a pass computes from the step's values is computed in the graph
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                self.logits = runner.model.forward(self.step, runner.slots)
-            self.graph = graph
+            self.graph, self.logits = _capture(lambda: parts.model.forward(self.step, parts.slots))
         self.graph.replay()
         return self.logits[:len(entries)]
+
+
+def _capture(work):
+    """Capture ``work()`` into a graph; returns ``(graph, what work returned)``.
+
+    Garbage that holds an older graph is collected before the capture begins and the cycle
+    collector stays off until it has ended: no graph's destructor may run in between."""
+    gc.collect()
+    was_on = gc.isenabled()
+    gc.disable()
+    try:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out = work()
+    finally:
+        if was_on:
+            gc.enable()
+    return graph, out
+
+
+class _RunnerParts:
+    """What a graph needs of the runner it belongs to, without the runner itself (which owns
+    the graphs: a reference back would make a cycle that only the collector could free)."""
+
+    def __init__(self, runner):
+        self.model = runner.model
+        self.cache = runner.cache
+        self.slots = runner.slots
+        self.device = runner.device
+        self.dtype = runner.dtype
+        self.pad_state_slot = runner.pad_state_slot
+        self.max_blocks_per_seq = runner.ecfg.max_blocks_per_seq
+        self.max_num_seqs = runner.ecfg.max_num_seqs
 
 
 class DecodeGraphs:
     """The graphs of a runner, keyed by (batch bucket, context bucket)."""
 
     def __init__(self, runner, max_graphs: int = 32):
-        self.runner = runner
+        self.parts = _RunnerParts(runner)
         self.max_graphs = max_graphs
         self.graphs: Dict[Tuple[int, int], _Graph] = {}
+
+    def close(self) -> None:
+        """Drop every captured graph, after the device has finished what it was given."""
+        if self.graphs:
+            if torch.cuda.is_available():
+                torch.cuda.synchronize()
+            self.graphs.clear()
 
     @staticmethod
     def takes(entries: Sequence[StepEntry]) -> bool:
@@ -184,10 +231,12 @@ class DecodeGraphs:
 
     def run(self, entries: Sequence[StepEntry], device_tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
         ctx = max(e.start for e in entries) + 1
-        key = (_batch_bucket(len(entries), self.runner.ecfg.max_num_seqs), _bucket(ctx))
+        key = (_batch_bucket(len(entries), self.parts.max_num_seqs), _bucket(ctx))
         g = self.graphs.get(key)
         if g is None:
             if len(self.graphs) >= self.max_graphs:
-                self.graphs.pop(next(iter(self.graphs)))
-            g = self.graphs[key] = _Graph(self.runner, *key)
+                # the oldest graph goes, here and now (nothing else refers to it), outside any capture
+                torch.cuda.synchronize()
+                del self.graphs[next(iter(self.graphs))]
+            g = self.graphs[key] = _Graph(self.parts, *key)
         return g.run(entries, device_tokens)

@@ -45,6 +45,16 @@ class LLM:
         self.runner = ModelRunner(self.model, self.engine_config)
         self.engine = LLMEngine(self.runner, self.engine_config)
 
+    def close(self) -> None:
+        """Give the captured decode graphs back now; ``with LLM(...) as llm:`` does it on leaving."""
+        self.runner.close()
+
+    def __enter__(self) -> "LLM":
+        return self
+
+    def __exit__(self, *exc) -> None:
+        self.close()
+
     def generate(self, prompts: Sequence[Sequence[int]],
                  params: Union[SamplingParams, Sequence[SamplingParams], None] = None) -> List[RequestOutput]:
         """Generate for every prompt (lists of token ids); results in the order of the prompts."""
@@ -53,7 +63,5 @@ class LLM:
         if len(params) != len(prompts):
             raise ValueError("one SamplingParams per prompt is needed")
         ids = [self.engine.add_request(p, sp) for p, sp in zip(prompts, params)]
-        already = len(self.engine.finished)
-        self.engine.run_until_complete()
-        by_id = {o.seq_id: o for o in self.engine.finished[already:]}
+        by_id = {o.seq_id: o for o in self.engine.run_until_complete()}
         return [by_id[i] for i in ids]

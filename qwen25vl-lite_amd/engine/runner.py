@@ -60,6 +60,12 @@ class ModelRunner:
             from .graph import DecodeGraphs
             self.graphs = DecodeGraphs(self)
 
+    def close(self) -> None:
+        """Drop the captured decode graphs now (after a device synchronization) instead of when the
+        runner goes away.  The runner keeps working: graphs are captured again when needed."""
+        if self.graphs is not None:
+            self.graphs.close()
+
     # ------------------------------------------------------------------ requests
     def admit(self, req_id) -> int:
         return self.cache.admit(req_id)

@@ -107,9 +107,9 @@ class LLMEngine:
         self.ecfg = engine_cfg or runner.ecfg
         self.waiting: Deque[Sequence_] = deque()
         self.running: List[Sequence_] = []
-        self.finished: List[RequestOutput] = []
         self.stats_ = EngineStats()
         self._next_id = 0
+        self._finished_total = 0
         self._ahead: Optional[Tuple[List[Tuple[Sequence_, int]], List[StepEntry], object]] = None
         self.position_rows = getattr(runner, "position_rows", 3)
 
@@ -317,7 +317,7 @@ class LLMEngine:
                 tokens = self.runner.sample(logits, *args)
             for seq, token in zip(sampled, tokens):
                 self._accept(seq, int(token), done)
-        self.finished.extend(done)
+        self._finished_total += len(done)
         return done
 
     # ------------------------------------------------------------------ looking one step ahead
@@ -398,11 +398,14 @@ class LLMEngine:
     # ------------------------------------------------------------------ driver
     def run_until_complete(self, max_steps: int = 100_000, max_stall: int = 64) -> List[RequestOutput]:
         """Drive the engine until every request has finished; raise if the scheduler spins
-        without computing anything (reference engine.py:878-914)."""
+        without computing anything (reference engine.py:878-914).  Returns the requests that finished
+        during this call (the engine keeps no list of them: a caller that drives :meth:`step` itself
+        gets each step's own)."""
         steps = stall = 0
+        finished: List[RequestOutput] = []
         last = self._progress()
         while self.has_work() and steps < max_steps:
-            self.step()
+            finished.extend(self.step())
             steps += 1
             now = self._progress()
             if now == last:
@@ -414,10 +417,10 @@ class LLMEngine:
                 stall, last = 0, now
         if self.has_work():
             raise RuntimeError(f"engine did not finish within {max_steps} steps")
-        return self.finished
+        return finished
 
     def _progress(self) -> tuple:
-        return (len(self.waiting), len(self.running), len(self.finished), self.stats_.batched_tokens,
+        return (len(self.waiting), len(self.running), self._finished_total, self.stats_.batched_tokens,
                 self.stats_.preemptions)
 
     def stats(self) -> Dict[str, float]:

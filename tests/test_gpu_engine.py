@@ -59,6 +59,43 @@ def test_long_decode_and_preemption(model_dirs):
     assert llm.runner.cache.pages_in_use() == [0, 0]
 
 
+def test_a_dropped_engine_frees_its_graphs_at_once(model_dirs):
+    """Captured graphs go when their engine goes, by reference count (the collector is off here):
+    a graph that lingered until a collection could be destroyed inside a later capture, which ends
+    the process.  A second and third engine then capture their own graphs."""
+    import gc
+    import weakref
+
+    from qwen25vl_lite_amd import LLM, SamplingParams
+
+    d = model_dirs["A"]
+    params = SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True)
+    first = None
+    for _ in range(3):
+        gc.collect()
+        gc.disable()
+        try:
+            llm = LLM(d, dtype="float32", num_blocks=16, block_size=16, max_num_seqs=2, hip_graph=True,
+                      enable_prefix_cache=False)
+            out = llm.generate([[1, 2, 3]], params)[0].output_token_ids
+            graphs = list(llm.runner.graphs.graphs.values())
+            assert graphs and all(g.graph is not None for g in graphs)
+            watched = [weakref.ref(g) for g in graphs] + [weakref.ref(g.graph) for g in graphs]
+            del graphs
+            torch.cuda.synchronize()
+            del llm
+            assert all(w() is None for w in watched), "a captured graph outlived its engine"
+        finally:
+            gc.enable()
+        first = first or out
+        assert out == first
+    with LLM(d, dtype="float32", num_blocks=16, block_size=16, max_num_seqs=2, hip_graph=True) as llm:
+        assert llm.generate([[1, 2, 3]], params)[0].output_token_ids == first
+        held = llm.runner.graphs
+        assert held.graphs
+    assert held.graphs == {}, "leaving the with block gives the graphs back"
+
+
 @pytest.mark.parametrize("name", ["B_sharp", "C_sharp"])
 def test_very_long_decode(model_dirs, name):
     """Three hundred tokens decoded from a short prompt, from HIP graphs: a dozen and a half pages,
@@ -149,14 +186,15 @@ def test_decode_step_queued_ahead_changes_nothing(model_dirs, name, dtype):
         for p, sp in zip(prompts[:3], params[:3]):
             engine.add_request(p, sp)
         steps = queued = 0
+        finished = []
         while engine.has_work():
-            engine.step()
+            finished += engine.step()
             steps += 1
             queued += engine._ahead is not None
             if steps == 6:            # three more arrive while the first three decode
                 for p, sp in zip(prompts[3:], params[3:]):
                     engine.add_request(p, sp)
-        outs = sorted(engine.finished, key=lambda o: o.seq_id)
+        outs = sorted(finished, key=lambda o: o.seq_id)
         assert runner.cache.pages_in_use() == [0] * len(runner.cache.groups)
         runner.cache.check()
         return [(o.output_token_ids, o.finish_reason) for o in outs], steps, queued

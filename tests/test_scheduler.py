@@ -28,8 +28,30 @@ class FakeRunner:
         self.cache = CacheManager(groups, ecfg.num_blocks, ecfg.block_size, ecfg.max_num_seqs,
                                   enable_prefix_cache=ecfg.enable_prefix_cache)
         self.batches = []
+        self.ahead_steps = 0
 
-    def execute(self, entries):
+    def decodes_from_graph(self, entries):
+        return bool(self.ecfg.hip_graph) and all(len(e.tokens) == 1 and e.positions is None and list(e.want) == [0]
+                                                 for e in entries)
+
+    def sample_begin(self, logits, params, prev_ids, steps):
+        ids = self.sample(logits, params, prev_ids, steps)
+
+        class Pending:
+            device_ids = torch.tensor(ids, dtype=torch.int32)
+
+            @staticmethod
+            def result():
+                return ids
+        return Pending
+
+    def execute(self, entries, device_tokens=None):
+        if device_tokens is not None:
+            # a step queued ahead: its token ids are still "on the device"
+            assert self.decodes_from_graph(entries) and len(device_tokens) == len(entries)
+            self.ahead_steps += 1
+            entries = [type(e)(req_id=e.req_id, tokens=[int(t)], start=e.start, want=e.want, positions=e.positions,
+                               rope_delta=e.rope_delta) for e, t in zip(entries, device_tokens)]
         rows = []
         total = 0
         seen = set()
@@ -251,3 +273,112 @@ def test_stall_guard():
     eng._schedule = lambda: []          # a scheduler that never runs anything
     with pytest.raises(RuntimeError):
         eng.run_until_complete(max_stall=5)
+
+
+# ---------------------------------------------------------------------------------------------
+# The decode step queued ahead (with decode graphs): whatever happens meanwhile, tokens and finish
+# reasons are those of an engine that schedules every step with the tokens known.
+
+def _both_ways(requests, arrivals=(), **kw):
+    """Run the same requests with and without the look-ahead; ``arrivals`` are ``(after step,
+    prompt, params)`` added while the engine runs.  Returns ``(outputs by id, engine, runner)`` of
+    each way."""
+    ways = []
+    for ahead in (False, True):
+        eng, runner = _engine(hip_graph=True, decode_lookahead=ahead, **kw)
+        for prompt, params in requests:
+            eng.add_request(prompt, params)
+        late = sorted(arrivals, key=lambda a: a[0])
+        outs, steps = {}, 0
+        while eng.has_work() or late:
+            while late and late[0][0] <= steps:
+                _, prompt, params = late.pop(0)
+                eng.add_request(prompt, params)
+            for o in eng.step():
+                outs[o.seq_id] = (o.output_token_ids, o.finish_reason)
+            steps += 1
+            assert steps < 2000
+        runner.cache.check()
+        if runner.cache.prefix_cache is not None:
+            runner.cache.prefix_cache.clear()      # what the remembered prompts hold
+            runner.cache.check()
+        assert all(n == 0 for n in runner.cache.pages_in_use()), "every page has come back"
+        assert eng._ahead is None
+        ways.append((outs, eng, runner))
+    assert ways[0][2].ahead_steps == 0
+    return ways
+
+
+def test_ahead_stop_token_found_one_step_late():
+    # request 0 stops on token 9 after four tokens, request 1 on the end-of-sequence token, request 2 by
+    # length: the first two are found out after the next step has been queued with a row for them
+    reqs = [([5], SamplingParams(max_tokens=20, ignore_eos=True, stop_token_ids=[9])),
+            ([20], SamplingParams(max_tokens=20)),
+            ([30], SamplingParams(max_tokens=12, ignore_eos=True))]
+    (plain, _, _), (ahead, eng, runner) = _both_ways(reqs, eos=27, enable_prefix_cache=False)
+    assert ahead == plain
+    assert ahead[0] == ([6, 7, 8, 9], "stop") and ahead[1][1] == "stop" and ahead[2][1] == "length"
+    assert runner.ahead_steps >= 8, "the look-ahead ran"
+    # a row computed for nothing is not counted as a decoded token
+    assert eng.stats()["decode_tokens"] == sum(len(t) for t, _ in ahead.values()) - 3
+
+
+def test_ahead_with_an_arrival_while_a_step_is_queued():
+    reqs = [([5, 6, 7], SamplingParams(max_tokens=10, ignore_eos=True))]
+    late = [(4, [40, 41], SamplingParams(max_tokens=5, ignore_eos=True)),
+            (5, [11] * 20, SamplingParams(max_tokens=3, ignore_eos=True))]
+    (plain, _, _), (ahead, _, runner) = _both_ways(reqs, late, enable_prefix_cache=False)
+    assert ahead == plain and len(ahead) == 3
+    assert runner.ahead_steps > 0
+
+
+def test_ahead_when_everyone_in_the_queued_step_has_finished():
+    # both stop on the same step through a stop token: the queued step holds only dead rows
+    reqs = [([5], SamplingParams(max_tokens=20, ignore_eos=True, stop_token_ids=[8])),
+            ([15], SamplingParams(max_tokens=20, ignore_eos=True, stop_token_ids=[18]))]
+    late = [(6, [1, 2], SamplingParams(max_tokens=2, ignore_eos=True))]
+    (plain, _, _), (ahead, eng, runner) = _both_ways(reqs, late, enable_prefix_cache=False)
+    assert ahead == plain and ahead[0] == ([6, 7, 8], "stop") and ahead[1] == ([16, 17, 18], "stop")
+    assert runner.ahead_steps > 0
+
+
+def test_ahead_when_pages_run_out_while_queueing():
+    # five pages: both requests need a third page for the same step; the first gets the last free page
+    # inside the look-ahead, the second does not: the queued step is given up and the scheduler,
+    # with the tokens known, preempts as it would have
+    reqs = [([(3 * j) % VOCAB for j in range(31)], SamplingParams(max_tokens=8, ignore_eos=True)),
+            ([(5 * j) % VOCAB for j in range(31)], SamplingParams(max_tokens=8, ignore_eos=True))]
+    (plain, e0, _), (ahead, e1, runner) = _both_ways(reqs, num_blocks=5, enable_prefix_cache=False)
+    assert ahead == plain
+    assert e0.stats()["preemptions"] >= 1 and e1.stats()["preemptions"] >= 1
+    for (prompt, _), (tokens, reason) in zip(reqs, (ahead[0], ahead[1])):
+        assert tokens == _expected(prompt, 8) and reason == "length"
+
+
+def test_ahead_with_the_prefix_cache():
+    shared = [(7 * i) % VOCAB for i in range(40)]
+    reqs = [(shared + [1], SamplingParams(max_tokens=6, ignore_eos=True)),
+            (shared + [2, 3], SamplingParams(max_tokens=4, ignore_eos=True, stop_token_ids=[5]))]
+    late = [(9, shared + [9], SamplingParams(max_tokens=5, ignore_eos=True)),
+            (12, shared[:32], SamplingParams(max_tokens=3, ignore_eos=True))]
+    (plain, e0, _), (ahead, e1, runner) = _both_ways(reqs, late, max_num_seqs=2)
+    assert ahead == plain and runner.ahead_steps > 0
+    assert e1.stats()["prefix_cache_tokens_saved"] == e0.stats()["prefix_cache_tokens_saved"] > 0
+
+
+def test_ahead_is_left_alone_by_penalties_and_by_waiting_requests():
+    reqs = [([5], SamplingParams(max_tokens=6, ignore_eos=True, repetition_penalty=1.3))]
+    (plain, _, _), (ahead, _, runner) = _both_ways(reqs, enable_prefix_cache=False)
+    assert ahead == plain and runner.ahead_steps == 0, "a sampler that reads the generated tokens waits for them"
+    reqs = [([i + 1], SamplingParams(max_tokens=6, ignore_eos=True)) for i in range(3)]
+    (plain, _, _), (ahead, _, runner) = _both_ways(reqs, max_num_seqs=2, enable_prefix_cache=False)
+    assert ahead == plain
+
+
+def test_finished_outputs_are_handed_over_once():
+    eng, _ = _engine()
+    eng.add_request([1, 2], SamplingParams(max_tokens=2, ignore_eos=True))
+    assert len(eng.run_until_complete()) == 1
+    eng.add_request([3, 4], SamplingParams(max_tokens=2, ignore_eos=True))
+    outs = eng.run_until_complete()
+    assert len(outs) == 1 and outs[0].prompt_token_ids == [3, 4]
