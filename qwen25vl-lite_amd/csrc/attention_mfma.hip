@@ -23,6 +23,8 @@
 // registers, and merge through LDS; for very long contexts the keys are further split among
 // blocks, whose partial sums a second kernel merges.
 #include "common.h"
+#include "attention_mfma.h"
+#include <mutex>
 
 #ifndef HD
 #error "compile with -DHD=<head size>"
@@ -859,10 +861,10 @@ extern "C" long long qvl_attn_mfma_scratch_floats(int num_tiles, int nkv, int ns
   return (long long)num_tiles * nkv * nsplit * PART_STRIDE;
 }
 
-extern "C" int qvl_attn_mfma_coop(const void* q, const void* kc, const void* vc, const void* bt, int table_width,
-                                  const void* cu_q, const void* ctx_len, const void* tile_req, const void* tile_ct,
-                                  int num_tiles, void* out, void* scratch, int nq, int nkv, int ps, int window,
-                                  float scale, int nsplit, int keys_per_split, hipStream_t stream) {
+static int launch_coop(const void* q, const void* kc, const void* vc, const void* bt, int table_width,
+                       const void* cu_q, const void* ctx_len, const void* tile_req, const void* tile_ct,
+                       int num_tiles, void* out, void* scratch, int nq, int nkv, int ps, int window, float scale,
+                       int nsplit, int keys_per_split, hipStream_t stream) {
   const int c = check_common(num_tiles, nq, nkv, ps, table_width);
   if (c >= 0) return c;
   if (nsplit <= 0 || nsplit > 65535 || (nsplit > 1 && (keys_per_split <= 0 || keys_per_split % 32 || !scratch)))
@@ -877,4 +879,67 @@ extern "C" int qvl_attn_mfma_coop(const void* q, const void* kc, const void* vc,
     hipLaunchKernelGGL(attn_mfma_merge_kernel, dim3(num_tiles, nkv), dim3(256), 0, stream, (const float*)scratch,
                        (const int*)cu_q, (const int*)tile_req, (const int*)tile_ct, (bf16_t*)out, nq, nkv, nsplit);
   return qvl_launch_status();
+}
+
+extern "C" int qvl_attn_mfma_coop(const void* q, const void* kc, const void* vc, const void* bt, int table_width,
+                                  const void* cu_q, const void* ctx_len, const void* tile_req, const void* tile_ct,
+                                  int num_tiles, void* out, void* scratch, int nq, int nkv, int ps, int window,
+                                  float scale, int nsplit, int keys_per_split, hipStream_t stream) {
+  return launch_coop(q, kc, vc, bt, table_width, cu_q, ctx_len, tile_req, tile_ct, num_tiles, out, scratch, nq, nkv,
+                     ps, window, scale, nsplit, keys_per_split, stream);
+}
+
+// ---------------------------------------------------------------------------------------------
+// The same attention with the partial results of a split call in memory the library owns: the
+// call allocates nothing (see attention_mfma.h).  The array below exists once per GPU the library
+// runs on, for the life of the process.  In host code its name is only a handle: the device
+// address is asked for once per device and kept, and only that address is ever handed to a kernel.
+static __device__ __align__(256) float scratch[QVL_ATTN_STATIC_SCRATCH_FLOATS];
+
+#define QVL_MAX_DEVICES 64
+static float* scratch_of_device[QVL_MAX_DEVICES];
+static std::mutex scratch_lock;
+
+// The current device's copy of the array, or nullptr (then *err says why).
+static float* static_scratch(int* err) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= QVL_MAX_DEVICES) {
+    *err = QVL_ERR_LIMIT;
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> hold(scratch_lock);
+  if (!scratch_of_device[dev]) {
+    float* ptr = nullptr;
+    if (hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) {
+      (void)hipGetLastError();
+      *err = QVL_ERR_LAUNCH;
+      return nullptr;
+    }
+    scratch_of_device[dev] = ptr;
+  }
+  return scratch_of_device[dev];
+}
+
+extern "C" long long qvl_attn_mfma_static_scratch_floats() { return QVL_ATTN_STATIC_SCRATCH_FLOATS; }
+
+extern "C" int qvl_attn_mfma_coop_static_init() {
+  int err = QVL_OK;
+  return static_scratch(&err) ? QVL_OK : err;
+}
+
+extern "C" int qvl_attn_mfma_coop_static(const void* q, const void* kc, const void* vc, const void* bt,
+                                         int table_width, const void* cu_q, const void* ctx_len,
+                                         const void* tile_req, const void* tile_ct, int num_tiles, void* out, int nq,
+                                         int nkv, int ps, int window, float scale, int nsplit, int keys_per_split,
+                                         hipStream_t stream) {
+  if (num_tiles < 0 || nkv <= 0 || nsplit <= 0) return QVL_ERR_SHAPE;
+  if (nsplit > 1 && qvl_attn_mfma_scratch_floats(num_tiles, nkv, nsplit) > QVL_ATTN_STATIC_SCRATCH_FLOATS)
+    return QVL_ERR_LIMIT;   // more partial results than the array holds: use qvl_attn_mfma_coop
+  int err = QVL_OK;
+  float* ptr = static_scratch(&err);
+  if (!ptr) return err;
+  // Every (tile, head, split) block writes all of its part before the merge kernel reads it, so
+  // nothing of the array has to start at zero, whatever the call before left there.
+  return launch_coop(q, kc, vc, bt, table_width, cu_q, ctx_len, tile_req, tile_ct, num_tiles, out, ptr, nq, nkv, ps,
+                     window, scale, nsplit, keys_per_split, stream);
 }

@@ -75,7 +75,8 @@ def _hipcc() -> Optional[str]:
 
 def _digest(source: str, defines: Mapping[str, object]) -> str:
     h = hashlib.sha1()
-    for path in (os.path.join(csrc_dir(), "common.h"), source):
+    headers = sorted(os.path.join(csrc_dir(), f) for f in os.listdir(csrc_dir()) if f.endswith(".h"))
+    for path in (*headers, source):
         with open(path, "rb") as fh:
             h.update(fh.read())
     stem = os.path.splitext(os.path.basename(source))[0]
