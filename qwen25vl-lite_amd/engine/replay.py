@@ -40,11 +40,12 @@ class Replayer:
         run_dtype = dtype_from_name(dtype)
         model = build_model(cfg, run_dtype, "cuda:0")
         load_weights(model_dir, model)
-        if ROUND_TO % block_size:
-            raise ValueError(f"block_size must divide {ROUND_TO}")
         max_tokens = max(ROUND_TO, (int(max_tokens) + ROUND_TO - 1) // ROUND_TO * ROUND_TO)
+        # Pages for max_tokens tokens; a page size that does not divide the rounding unit can leave
+        # each live request one page short of that, so it gets one more per request.
+        num_blocks = (max_tokens + block_size - 1) // block_size + (max_live if ROUND_TO % block_size else 0)
         ecfg = EngineConfig(
-            num_blocks=max_tokens // block_size, block_size=block_size, max_num_seqs=max_live,
+            num_blocks=num_blocks, block_size=block_size, max_num_seqs=max_live,
             max_num_batched_tokens=max_tokens, max_model_len=max_tokens, enable_prefix_cache=False,
             dtype=run_dtype, device="cuda:0")
         self.runner = ModelRunner(model, ecfg)

@@ -97,12 +97,26 @@ def mixed_trace(requests: Dict[str, List[int]], seed: int = 0, max_live: int = 4
     return steps, peak
 
 
-def run_steps(replayer, steps: List[dict]) -> Dict[Tuple[str, int], torch.Tensor]:
-    """Replay and return {(request, index in its sequence): logits row} on the host."""
+def run_steps(replayer, steps: List[dict], holders: Dict[Tuple[int, int], set] = None
+              ) -> Dict[Tuple[str, int], torch.Tensor]:
+    """Replay and return {(request, index in its sequence): logits row} on the host.  ``holders``,
+    if given, collects for every (cache group, page) the requests that held it at some time."""
     at: Dict[str, int] = {}
     out: Dict[Tuple[str, int], torch.Tensor] = {}
+    cache = replayer.runner.cache
     for rec in steps:
+        if holders is not None:
+            # pages are handed out when the step runs and given back when a request ends: look before the ends
+            ends, rec = rec.get("end", []), dict(rec, end=[])
         logits = replayer.step(rec)
+        if holders is not None:
+            for e in rec["entries"]:
+                for g in range(len(cache.groups)):
+                    for page in cache.table(e["id"], g):
+                        if page >= 0:
+                            holders.setdefault((g, int(page)), set()).add(e["id"])
+            if ends:
+                replayer.step({"entries": [], "end": ends})
         rows = logits.float().cpu() if logits is not None else None
         k = 0
         for e in rec["entries"]:

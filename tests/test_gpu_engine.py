@@ -114,8 +114,10 @@ def test_very_long_decode(model_dirs, name):
     assert llm.runner.cache.pages_in_use() == [0] * len(llm.runner.cache.groups)
 
 
-@pytest.mark.parametrize("name, dtype", [("B_sharp", "float32"), ("C_sharp", "bfloat16"), ("A", "bfloat16")])
-def test_decode_from_hip_graphs_gives_the_same_tokens(model_dirs, name, dtype):
+@pytest.mark.parametrize("name, dtype, block_size", [("B_sharp", "float32", 16), ("C_sharp", "bfloat16", 16),
+                                                     ("A", "bfloat16", 16), ("B_sharp", "float32", 48),
+                                                     ("C_sharp", "bfloat16", 32)])
+def test_decode_from_hip_graphs_gives_the_same_tokens(model_dirs, name, dtype, block_size):
     """Decode steps replayed from HIP graphs, many replays with eager prefill steps, admissions and
     finishes in between (batch size and context bucket change): every token equals the eager run's."""
     from qwen25vl_lite_amd import LLM, SamplingParams
@@ -124,7 +126,7 @@ def test_decode_from_hip_graphs_gives_the_same_tokens(model_dirs, name, dtype):
     vocab = {"A": 256, "B": 509, "C": 300}[name[0]]
     prompts = [random_tokens(n, vocab, 50 + n) for n in (5, 250, 31, 70, 12)]
     params = [SamplingParams(temperature=0.0, max_tokens=m, ignore_eos=True) for m in (40, 30, 60, 9, 25)]
-    common = dict(dtype=dtype, num_blocks=64, block_size=16, max_num_seqs=3, max_num_batched_tokens=64,
+    common = dict(dtype=dtype, num_blocks=64, block_size=block_size, max_num_seqs=3, max_num_batched_tokens=64,
                   enable_prefix_cache=False)
     eager = LLM(d, **common).generate(prompts, params)
     llm = LLM(d, hip_graph=True, **common)
@@ -283,6 +285,70 @@ def test_everything_at_once(model_dirs, name, seed):
     llm.runner.cache.check()
     cached = len(llm.runner.cache.prefix_cache) if llm.runner.cache.prefix_cache else 0
     assert llm.runner.cache.pages_in_use()[0] == cached
+
+
+@pytest.mark.parametrize("name, seed, pool, seqs", [("A", 3, 14, 5), ("C", 6, 20, 3)])
+def test_look_ahead_under_preemption_stops_arrivals_and_the_prefix_cache(model_dirs, name, seed, pool, seqs):
+    """The decode step queued ahead, in a server's day: requests arriving over forty steps, a shared
+    prefix and the prefix cache (model A) or a windowed group (model C), stop tokens frequent enough
+    to end some requests early (found out one step late), seeded sampling beside greedy, a request
+    with a penalty, and so few pages that requests are preempted and computed again.  Tokens and
+    finish reasons are those of the engine without the look-ahead; greedy requests give the plain
+    implementation's tokens; all pages come back."""
+    import random
+    from qwen25vl_lite_amd import LLM, SamplingParams
+
+    d = model_dirs[name]
+    vocab = {"A": 256, "C": 300}[name]
+    rng = random.Random(1000 + seed)
+    n = 10
+    shared = random_tokens(36, vocab, 4000 + seed)
+    prompts = [random_tokens(rng.randint(2, 50), vocab, 5000 + 50 * seed + i) for i in range(n)]
+    for i in (0, 4, 7):
+        prompts[i] = shared + prompts[i][:12]
+    stop_pool = tuple(rng.randrange(vocab) for _ in range(12))
+    params = []
+    for i in range(n):
+        kind = rng.random()
+        params.append(SamplingParams(temperature=0.0 if kind < 0.6 else 0.9, top_k=0 if kind < 0.8 else 30,
+                                     seed=rng.randint(0, 99), max_tokens=rng.randint(2, 50), ignore_eos=True,
+                                     stop_token_ids=stop_pool if i % 2 else (),
+                                     repetition_penalty=1.2 if i == 5 else 1.0))
+    arrive = sorted(rng.randint(0, 40) for _ in range(n))
+    arrive[0] = 0
+
+    def run(look):
+        llm = LLM(d, dtype="float32", num_blocks=pool, block_size=16, max_num_seqs=seqs, max_num_batched_tokens=48,
+                  enable_prefix_cache=True, hip_graph=True, decode_lookahead=look)
+        eng, step, nxt, queued, outs = llm.engine, 0, 0, 0, []
+        while nxt < n or eng.has_work():
+            while nxt < n and arrive[nxt] <= step:
+                eng.add_request(prompts[nxt], params[nxt])
+                nxt += 1
+            if eng.has_work():
+                outs += eng.step()
+                queued += eng._ahead is not None
+            step += 1
+            assert step < 5000
+        cache = llm.runner.cache
+        cache.check()
+        cached = len(cache.prefix_cache) if cache.prefix_cache else 0
+        assert cache.pages_in_use()[0] == cached and all(u == 0 for u in cache.pages_in_use()[1:])
+        return sorted(((o.seq_id, o.output_token_ids, o.finish_reason) for o in outs)), queued, eng.stats()
+
+    plain, none_queued, stats0 = run(False)
+    ahead, queued, stats1 = run(True)
+    assert none_queued == 0 and queued > 10, queued
+    assert stats0["preemptions"] > 0 and stats1["preemptions"] > 0, (stats0, stats1)
+    assert any(reason == "stop" for _, _, reason in ahead)
+    if name == "A":
+        assert stats1["prefix_cache_hits"] > 0
+    assert ahead == plain
+    for sid, tokens, reason in ahead:
+        p = params[sid]
+        if p.temperature == 0.0 and p.repetition_penalty == 1.0:
+            want = _plain_greedy(d, prompts[sid], len(tokens))
+            assert tokens == want, sid
 
 
 @pytest.mark.parametrize("name", ["B_sharp", "C_sharp"])

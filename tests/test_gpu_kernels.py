@@ -51,11 +51,13 @@ def test_add_rmsnorm(width, delta_dtype, out_dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("nq, nkv, hd, sections", [(6, 2, 24, (4, 4, 4)), (5, 1, 48, (10, 6, 8)), (4, 4, 128, (16, 24, 24))])
-def test_rope_kv_write(dtype, nq, nkv, hd, sections):
+@pytest.mark.parametrize("nq, nkv, hd, sections, ps", [(6, 2, 24, (4, 4, 4), 16), (5, 1, 48, (10, 6, 8), 16),
+                                                       (4, 4, 128, (16, 24, 24), 16), (6, 2, 24, (4, 4, 4), 48),
+                                                       (4, 4, 128, (16, 24, 24), 32)])
+def test_rope_kv_write(dtype, nq, nkv, hd, sections, ps):
     from qwen25vl_lite_amd.ops import kernels
     torch.manual_seed(hd)
-    n, ps, pages, theta = 11, 16, 5, 1e4
+    n, pages, theta = 11, 5, 1e4
     x = torch.randn(n, (nq + 2 * nkv) * hd)
     bias = torch.randn((nq + 2 * nkv) * hd) * 0.1
     pos = torch.stack([torch.randint(0, 5000, (n,)) for _ in range(3)])
@@ -131,12 +133,11 @@ def _paged(k, v, ps, pages, dtype, seed):
 ATTN_SHAPES = [(6, 2, 24, None), (5, 1, 48, 40), (8, 8, 16, 7), (14, 2, 128, None), (4, 2, 80, 130)]
 
 
-def _attention_case(dtype, nq, nkv, hd, window, lens=(333, 17, 64, 1), qlens=(5, 17, 1, 1)):
+def _attention_case(dtype, nq, nkv, hd, window, lens=(333, 17, 64, 1), qlens=(5, 17, 1, 1), ps=16):
     """Prompt portions and single tokens of several requests in one call, pages shuffled, stale
     values in every unused slot.  One query and one far key are scaled so that a single score
     dominates: a kernel that misses that key (a page, a window edge) fails by far."""
     torch.manual_seed(nq * hd)
-    ps = 16
     lens, qlens = list(lens), list(qlens)   # context of each request after this step; its last qlen tokens are this step's
     last = lens[0] - 1
     k = [torch.randn(nkv, t, hd).to(dtype).float() for t in lens]
@@ -164,11 +165,16 @@ def _attention_case(dtype, nq, nkv, hd, window, lens=(333, 17, 64, 1), qlens=(5,
                 want=want, scale=scale, lens=lens, qlens=qlens)
 
 
+# other page sizes than 16 (the reference tests 32, reference tests/test_paged_attn_kernel.py:89);
+# 48 is the one where a 32-key block straddles pages at changing places
+PAGE_SIZES = [(14, 2, 128, None, 32), (5, 1, 48, 40, 48), (4, 2, 80, 130, 64), (6, 2, 24, None, 32)]
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("nq, nkv, hd, window", ATTN_SHAPES)
-def test_paged_attention_generic(dtype, nq, nkv, hd, window):
+@pytest.mark.parametrize("nq, nkv, hd, window, ps", [(*s, 16) for s in ATTN_SHAPES] + PAGE_SIZES)
+def test_paged_attention_generic(dtype, nq, nkv, hd, window, ps):
     from qwen25vl_lite_amd.ops import kernels
-    c = _attention_case(dtype, nq, nkv, hd, window)
+    c = _attention_case(dtype, nq, nkv, hd, window, ps=ps)
     out = kernels.paged_attention_generic(c["q"], c["kc"], c["vc"], c["table"], c["req"], c["seqpos"], nq, window,
                                           c["scale"])
     tol = dict(atol=2e-5, rtol=1e-4) if dtype == torch.float32 else dict(atol=1.5e-2, rtol=2e-2)
@@ -176,14 +182,15 @@ def test_paged_attention_generic(dtype, nq, nkv, hd, window):
 
 
 @pytest.mark.parametrize("split", ["tile", "tile_two_groups", "coop", "coop_split"])
-@pytest.mark.parametrize("nq, nkv, hd, window", [s for s in ATTN_SHAPES if s[2] % 16 == 0])
-def test_paged_attention_matrix_cores(nq, nkv, hd, window, split, monkeypatch):
+@pytest.mark.parametrize("nq, nkv, hd, window, ps", [(*s, 16) for s in ATTN_SHAPES if s[2] % 16 == 0]
+                         + [s for s in PAGE_SIZES if s[2] % 16 == 0])
+def test_paged_attention_matrix_cores(nq, nkv, hd, window, ps, split, monkeypatch):
     """The matrix-core kernels on the same case: blocks that own several tiles and share the keys
     through LDS (one group of waves, or two that take the key blocks in turn and merge), the waves
     of a block sharing one tile, and the keys further split among blocks."""
     from qwen25vl_lite_amd.ops import attention_mfma
     from qwen25vl_lite_amd.parts import StepContext
-    c = _attention_case(torch.bfloat16, nq, nkv, hd, window)
+    c = _attention_case(torch.bfloat16, nq, nkv, hd, window, ps=ps)
     plan = {"tile": ("tile", 1, 0), "tile_two_groups": ("tile", 1, 0), "coop": ("coop", 1, 0),
             "coop_split": ("coop", 6, 64)}[split]
     groups = {"tile": 1, "tile_two_groups": 2}.get(split)
@@ -206,15 +213,17 @@ def test_paged_attention_matrix_cores(nq, nkv, hd, window, split, monkeypatch):
     assert torch.allclose(out.float().cpu(), c["want"], atol=1.5e-2, rtol=2e-2), err
 
 
-@pytest.mark.parametrize("nq, nkv, hd, window", [(28, 4, 128, None), (6, 2, 48, 100), (4, 4, 256, 257), (5, 1, 16, None)])
-def test_paged_attention_long_portions(nq, nkv, hd, window):
+@pytest.mark.parametrize("nq, nkv, hd, window, ps", [(28, 4, 128, None, 16), (6, 2, 48, 100, 16), (4, 4, 256, 257, 16),
+                                                     (5, 1, 16, None, 16), (28, 4, 128, None, 48), (6, 2, 48, 100, 32),
+                                                     (4, 4, 256, 257, 64)])
+def test_paged_attention_long_portions(nq, nkv, hd, window, ps):
     """Prompt portions long enough for several blocks of several waves per request, next to a
     short portion and a decoded token: the kernel that shares keys through LDS walks the union of
     its waves' ranges, with blocks that some of its waves skip."""
     from qwen25vl_lite_amd.ops import attention_mfma, kernels
     from qwen25vl_lite_amd.parts import StepContext
     lens, qlens = (413, 150, 90), (380, 3, 1)
-    c = _attention_case(torch.bfloat16, nq, nkv, hd, window, lens, qlens)
+    c = _attention_case(torch.bfloat16, nq, nkv, hd, window, lens, qlens, ps=ps)
     cu = [0]
     for ql in qlens:
         cu.append(cu[-1] + ql)
@@ -373,18 +382,19 @@ def test_no_cpu_path():
         kernels.swiglu(torch.zeros(2, 4, dtype=torch.float16).cuda())
 
 
+@pytest.mark.parametrize("ps", [16, 32, 48])
 @pytest.mark.parametrize("m, nq, nkv, hd, k, bias, lazy", [(1, 4, 2, 16, 64, True, False), (8, 28, 4, 128, 3584, True, True),
                                                          (16, 6, 3, 48, 136, False, True), (5, 3, 0, 80, 104, True, False),
                                                          (32, 28, 4, 128, 3584, True, True), (17, 6, 3, 48, 136, False, True),
                                                          (27, 4, 2, 16, 64, True, False)])
-def test_projection_with_rotation_and_cache_write_folded_in(m, nq, nkv, hd, k, bias, lazy):
+def test_projection_with_rotation_and_cache_write_folded_in(m, nq, nkv, hd, k, bias, lazy, ps):
     """The stacked q | k | v projection of a few rows that rotates and stores inside the product's
     kernel equals the product followed by the rotation kernel: queries, and every slot of the
     cache (the slots of other tokens keep their stale values)."""
     from qwen25vl_lite_amd.ops import kernels, skinny
     from qwen25vl_lite_amd.ops.linear import linear
     torch.manual_seed(hd + m)
-    ps, pages = 16, 7
+    pages = 7
     n_out = (nq + 2 * nkv) * hd
     w = (torch.randn(n_out, k) / math.sqrt(k)).bfloat16().cuda()
     b = torch.randn(n_out).cuda() if bias else None

@@ -8,7 +8,8 @@ from replay_util import (mixed_trace, portion_trace, random_tokens, round64, run
 
 pytestmark = pytest.mark.gpu
 
-LENGTHS = {"A": [5, 17, 33, 70], "B": [1, 9, 40, 64, 97], "C": [3, 48, 81, 130]}
+# more requests than the mixed trace keeps live (four), so that pages freed inside it go to later ones
+LENGTHS = {"A": [5, 17, 33, 70, 12, 41], "B": [1, 9, 40, 64, 97], "C": [3, 48, 81, 130, 20, 66]}
 VOCAB = {"A": 256, "B": 509, "C": 300}
 
 
@@ -44,14 +45,21 @@ def _compare(got, ref, dtype, what, bound=None):
     return worst
 
 
-def _replayer(model_dir, dtype, max_tokens):
+def _replayer(model_dir, dtype, max_tokens, block_size=16):
     from qwen25vl_lite_amd.engine.replay import Replayer
-    return Replayer(model_dir, dtype, max_tokens)
+    return Replayer(model_dir, dtype, max_tokens, block_size)
+
+
+# every model with pages of 16 tokens; the sharp ones (a wrong key shows) also with pages of 32, 48
+# (a page size that divides neither the 64-token rounding nor a 32-key block evenly) and 64
+EVERY_WAY = [(n, 16) for n in ("A", "B", "C", "A_sharp", "B_sharp", "C_sharp")] + \
+            [("A_sharp", 32), ("B_sharp", 48), ("C_sharp", 32), ("C_sharp", 48), ("B_sharp", 64), ("C_sharp", 64)]
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "A_sharp", "B_sharp", "C_sharp"])
-def test_replay_every_way(model_dirs, name, dtype):
+@pytest.mark.parametrize("name, block_size", EVERY_WAY)
+def test_replay_every_way(model_dirs, name, dtype, block_size):
+    _replayer = lambda d, dt, n: globals()["_replayer"](d, dt, n, block_size)
     d = model_dirs[name]
     requests = _requests(name)
     ref = _reference(d, requests, dtype)
@@ -77,9 +85,12 @@ def test_replay_every_way(model_dirs, name, dtype):
 
     steps, peak = mixed_trace(requests, seed=7)
     rp = _replayer(d, dtype, peak)
-    got = run_steps(rp, steps)
+    holders = {}
+    got = run_steps(rp, steps, holders)
     assert len(got) == total
     print(name, dtype, "mixed", _compare(got, ref, dtype, "mixed"), "pool tokens", peak)
+    reused = sum(len(who) > 1 for who in holders.values())
+    assert reused >= 2, "the trace must hand pages of finished requests to later ones"
     rp.runner.cache.check()
     assert rp.runner.cache.pages_in_use() == [0] * len(rp.runner.cache.groups)
 
