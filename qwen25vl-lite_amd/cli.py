@@ -22,7 +22,7 @@ __all__ = ["main", "build_parser"]
 
 
 def _llm(args):
-    from .config import Qwen25VLConfig
+    from .config import load_config
     from .engine.llm import LLM
 
     if "cuda" not in args.device:
@@ -35,7 +35,7 @@ def _llm(args):
         preemption=args.preemption, hip_graph=args.cuda_graph, decode_lookahead=args.decode_lookahead)
     t0 = time.time()
     if args.random_weights is not None:
-        llm = LLM(Qwen25VLConfig.from_pretrained(args.model), args.dtype, random_seed=args.random_weights,
+        llm = LLM(load_config(args.model), args.dtype, random_seed=args.random_weights,
                   device=device, **options)
     else:
         llm = LLM(args.model, args.dtype, device=device, **options)
@@ -81,7 +81,7 @@ def cmd_bench(args) -> int:
     from .sampling.params import SamplingParams
 
     llm = _llm(args)
-    vocab = llm.config.vocab_size
+    vocab = llm.model.spec.vocab_size
     prompt = [(1000 + i) % vocab for i in range(args.prompt_tokens)]
     params = SamplingParams(temperature=0.0, max_tokens=args.max_tokens, ignore_eos=True)
     t0 = time.time()
@@ -103,10 +103,10 @@ def cmd_replay(args) -> int:
 
 
 def cmd_make_random(args) -> int:
-    from .config import Qwen25VLConfig, dtype_from_name
+    from .config import dtype_from_name, load_config
     from .weights import write_random_model
 
-    cfg = Qwen25VLConfig.from_pretrained(args.config)
+    cfg = load_config(args.config)
     write_random_model(cfg, args.out, args.seed, std=args.std, dtype=dtype_from_name(args.dtype))
     print(f"wrote {args.out}/config.json and model.safetensors (seed {args.seed})")
     return 0

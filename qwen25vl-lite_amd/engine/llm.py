@@ -9,7 +9,7 @@ from __future__ import annotations
 
 from typing import List, Optional, Sequence, Union
 
-from ..config import EngineConfig, Qwen25VLConfig, dtype_from_name
+from ..config import EngineConfig, dtype_from_name, load_config
 from ..models import build_model
 from ..sampling.params import SamplingParams
 from ..weights import fill_random, load_weights
@@ -22,22 +22,24 @@ __all__ = ["LLM"]
 class LLM:
     """``LLM(model_dir, dtype="bfloat16", **engine options).generate(prompts, params)``.
 
-    ``model`` is a folder with ``config.json`` and ``model.safetensors``, or a
-    :class:`Qwen25VLConfig` together with ``random_seed`` for random weights drawn on the GPU.
-    Engine options are the fields of :class:`EngineConfig`.
+    ``model`` is a folder with ``config.json`` and ``model.safetensors``, or a configuration
+    object (of any registered architecture) together with ``random_seed`` for random weights
+    drawn on the GPU.  The architecture named in ``config.json`` decides how the rest of the
+    file is read and which model is built.  Engine options are the fields of :class:`EngineConfig`.
     """
 
-    def __init__(self, model: Union[str, Qwen25VLConfig], dtype="bfloat16", *, random_seed: Optional[int] = None,
+    def __init__(self, model, dtype="bfloat16", *, random_seed: Optional[int] = None,
                  device: str = "cuda:0", **engine_options):
         run_dtype = dtype_from_name(dtype)
-        if isinstance(model, Qwen25VLConfig):
+        from_folder = isinstance(model, (str, bytes)) or hasattr(model, "__fspath__")
+        if from_folder:
+            self.config = load_config(model)
+        else:
             self.config = model
             if random_seed is None:
                 raise ValueError("a configuration without a model folder needs random_seed")
-        else:
-            self.config = Qwen25VLConfig.from_pretrained(model)
         self.model = build_model(self.config, run_dtype, device)
-        if isinstance(model, Qwen25VLConfig) or random_seed is not None:
+        if random_seed is not None:
             fill_random(self.model, int(random_seed))
         else:
             load_weights(model, self.model)

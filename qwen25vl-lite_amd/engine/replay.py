@@ -23,7 +23,7 @@ from typing import Dict, IO, Optional
 
 import torch
 
-from ..config import EngineConfig, Qwen25VLConfig, dtype_from_name
+from ..config import EngineConfig, dtype_from_name, load_config
 from ..models import build_model
 from ..weights import load_weights
 from .batch import StepEntry
@@ -36,7 +36,7 @@ ROUND_TO = 64  # a request's token count is rounded up to a multiple of this whe
 
 class Replayer:
     def __init__(self, model_dir: str, dtype: str, max_tokens: int, block_size: int = 16, max_live: int = 8):
-        cfg = Qwen25VLConfig.from_pretrained(model_dir)
+        cfg = load_config(model_dir)
         run_dtype = dtype_from_name(dtype)
         model = build_model(cfg, run_dtype, "cuda:0")
         load_weights(model_dir, model)

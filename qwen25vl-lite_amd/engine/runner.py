@@ -36,8 +36,12 @@ class ModelRunner:
         self.vocab_size = model.spec.vocab_size
         self.eos_token_id = model.spec.eos_token_id
         groups = model.cache_groups()
+        # A cached prefix holds keys and values only.  A mixer with a state of its own would start
+        # a request that adopted one from a cleared state, not from the state after the prefix:
+        # with such a mixer in the model the prefix cache stays off.
+        has_state = any(need is not None for need in model.entry_state)
         self.cache = CacheManager(groups, engine_cfg.num_blocks, engine_cfg.block_size, engine_cfg.max_num_seqs,
-                                  enable_prefix_cache=engine_cfg.enable_prefix_cache,
+                                  enable_prefix_cache=engine_cfg.enable_prefix_cache and not has_state,
                                   max_prefix_nodes=max_prefix_nodes)
         self.storage = KVStorage(groups, engine_cfg.num_blocks, engine_cfg.block_size, self.dtype, self.device)
         # one state row per request slot, and a spare one that the padding rows of a captured

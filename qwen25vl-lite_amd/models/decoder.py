@@ -25,11 +25,15 @@ def _collect(part: Part, prefix: str, out: Dict[str, Tuple[Part, str, ParamSpec]
         _collect(sub, f"{prefix}{name}.", out)
 
 
-def _mixer_of(block: Block) -> Optional[Mixer]:
-    for sub in block.sub_parts().values():
+def _mixers_of(block: Part, prefix: str = "") -> List[Tuple[str, Mixer]]:
+    """Every mixer inside a block, however deep, with its dotted sub-part name."""
+    found: List[Tuple[str, Mixer]] = []
+    for name, sub in block.sub_parts().items():
         if isinstance(sub, Mixer):
-            return sub
-    return None
+            found.append((prefix + name, sub))
+        else:
+            found.extend(_mixers_of(sub, f"{prefix}{name}."))
+    return found
 
 
 class DecoderModel:
@@ -44,9 +48,13 @@ class DecoderModel:
         self.embed: Optional[torch.Tensor] = None
         self.head: Optional[torch.Tensor] = None
 
-        # the run list: which cache layer and state each entry owns
+        # The run list: which cache layer and state every mixer of every entry owns.  The lists
+        # below have one element per (run entry, mixer of its block), in run order ("places");
+        # entry_places[i] names the places of entry i by the mixer's sub-part name.  A block with
+        # one mixer, the usual case, has one place.
         self.group_needs: List[CacheNeed] = []
         self.group_layers: List[int] = []
+        self.entry_places: List[Dict[str, int]] = []
         self.entry_group: List[Optional[int]] = []
         self.entry_cache_layer: List[Optional[int]] = []
         self.entry_writes: List[bool] = []
@@ -54,34 +62,43 @@ class DecoderModel:
         for i, entry in enumerate(spec.run):
             if not 0 <= entry.layer < len(self.blocks):
                 raise ValueError(f"run entry {i} names layer {entry.layer}, which does not exist")
-            mixer = _mixer_of(self.blocks[entry.layer])
-            need = mixer.cache_need() if mixer is not None else None
-            self.entry_state.append(mixer.state_need() if mixer is not None else None)
-            if need is None:
-                if entry.cache_from is not None:
-                    raise ValueError(f"run entry {i} reads a cache but its mixer keeps none")
-                self.entry_group.append(None)
-                self.entry_cache_layer.append(None)
-                self.entry_writes.append(False)
-                continue
+            mixers = _mixers_of(self.blocks[entry.layer])
             if entry.cache_from is not None:
                 src = entry.cache_from
-                if not 0 <= src < i or self.entry_group[src] is None or not self.entry_writes[src]:
+                if not 0 <= src < i:
                     raise ValueError(f"run entry {i} must read the cache of an earlier entry that writes one")
-                if self.group_needs[self.entry_group[src]] != need:
-                    raise ValueError(f"run entry {i} reads the cache of entry {src}, whose shape or window differs")
-                self.entry_group.append(self.entry_group[src])
-                self.entry_cache_layer.append(self.entry_cache_layer[src])
-                self.entry_writes.append(False)
-                continue
-            if need not in self.group_needs:
-                self.group_needs.append(need)
-                self.group_layers.append(0)
-            g = self.group_needs.index(need)
-            self.entry_group.append(g)
-            self.entry_cache_layer.append(self.group_layers[g])
-            self.entry_writes.append(True)
-            self.group_layers[g] += 1
+                if not any(m.cache_need() is not None for _, m in mixers):
+                    raise ValueError(f"run entry {i} reads a cache but its mixer keeps none")
+            places: Dict[str, int] = {}
+            for name, mixer in mixers:
+                need = mixer.cache_need()
+                places[name] = len(self.entry_state)
+                self.entry_state.append(mixer.state_need())
+                if need is None:
+                    self.entry_group.append(None)
+                    self.entry_cache_layer.append(None)
+                    self.entry_writes.append(False)
+                    continue
+                if entry.cache_from is not None:
+                    src_place = self.entry_places[entry.cache_from].get(name)
+                    if src_place is None or self.entry_group[src_place] is None or not self.entry_writes[src_place]:
+                        raise ValueError(f"run entry {i} must read the cache of an earlier entry that writes one")
+                    if self.group_needs[self.entry_group[src_place]] != need:
+                        raise ValueError(
+                            f"run entry {i} reads the cache of entry {entry.cache_from}, whose shape or window differs")
+                    self.entry_group.append(self.entry_group[src_place])
+                    self.entry_cache_layer.append(self.entry_cache_layer[src_place])
+                    self.entry_writes.append(False)
+                    continue
+                if need not in self.group_needs:
+                    self.group_needs.append(need)
+                    self.group_layers.append(0)
+                g = self.group_needs.index(need)
+                self.entry_group.append(g)
+                self.entry_cache_layer.append(self.group_layers[g])
+                self.entry_writes.append(True)
+                self.group_layers[g] += 1
+            self.entry_places.append(places)
 
         self.params: Dict[str, Tuple[Optional[Part], str, ParamSpec]] = {}
         self.params[spec.embed_name] = (None, "embed", ParamSpec((spec.vocab_size, spec.hidden_size), "table"))
@@ -125,16 +142,25 @@ class DecoderModel:
         self.head = self.embed
 
     def make_slots(self, storage, state_tensors: List[Optional[torch.Tensor]]) -> List[LayerSlot]:
-        slots = []
-        for i in range(len(self.spec.run)):
-            g, layer = self.entry_group[i], self.entry_cache_layer[i]
-            slots.append(LayerSlot(
+        """One slot per run entry.  ``state_tensors`` has one element per place (see
+        ``entry_state``).  The slot of an entry is its first mixer's; a block with several
+        mixers finds each one's under the mixer's sub-part name in ``slot.by_part``."""
+        def place_slot(p: int) -> LayerSlot:
+            g, layer = self.entry_group[p], self.entry_cache_layer[p]
+            return LayerSlot(
                 group=g,
                 k_cache=storage.k[g][layer] if g is not None else None,
                 v_cache=storage.v[g][layer] if g is not None else None,
-                writes=self.entry_writes[i],
-                state=state_tensors[i],
-            ))
+                writes=self.entry_writes[p],
+                state=state_tensors[p],
+            )
+
+        slots = []
+        for places in self.entry_places:
+            by_part = {name: place_slot(p) for name, p in places.items()}
+            first = next(iter(by_part.values()), LayerSlot(writes=False))
+            first.by_part = by_part
+            slots.append(first)
         return slots
 
     # ------------------------------------------------------------------ the step

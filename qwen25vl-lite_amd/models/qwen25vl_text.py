@@ -15,9 +15,15 @@ from ..config.registry import register_architecture
 from ..parts.base import PartSpec
 from .spec import LayerSpec, ModelSpec, RunEntry
 
-__all__ = ["qwen25vl_text_spec", "map_checkpoint_name"]
+__all__ = ["qwen25vl_text_spec", "map_checkpoint_name", "store_checkpoint_name"]
 
 _ROOTS = ("embed_tokens", "layers", "norm")
+
+
+def store_checkpoint_name(name: str) -> str:
+    """Canonical name -> the released checkpoints' name (the inverse of :func:`map_checkpoint_name`
+    for the layout a written model folder uses)."""
+    return name if name.startswith("lm_head.") else "model.language_model." + name
 
 
 def map_checkpoint_name(name: str) -> Optional[str]:
@@ -90,10 +96,12 @@ def qwen25vl_text_spec(config: Qwen25VLConfig) -> ModelSpec:
         tie_word_embeddings=t.tie_word_embeddings,
         position_rows=3,
         map_name=map_checkpoint_name,
+        store_name=store_checkpoint_name,
         eos_token_id=config.eos_token_id,
     )
 
 
-register_architecture("Qwen2_5_VLForConditionalGeneration", qwen25vl_text_spec)
-register_architecture("qwen2_5_vl", qwen25vl_text_spec)        # model_type, for a config.json without architectures
-register_architecture("qwen2_5_vl_text", qwen25vl_text_spec)   # model_type of a bare text_config
+register_architecture("Qwen2_5_VLForConditionalGeneration", qwen25vl_text_spec, Qwen25VLConfig.from_dict)
+# model_type, for a config.json without architectures, and that of a bare text_config
+register_architecture("qwen2_5_vl", qwen25vl_text_spec, Qwen25VLConfig.from_dict)
+register_architecture("qwen2_5_vl_text", qwen25vl_text_spec, Qwen25VLConfig.from_dict)

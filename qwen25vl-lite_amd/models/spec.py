@@ -47,4 +47,6 @@ class ModelSpec:
     head_name: str = "lm_head.weight"
     # checkpoint tensor name -> canonical name, or None for a tensor this model ignores
     map_name: Callable[[str], Optional[str]] = field(default=lambda name: name)
+    # canonical name -> the name a written model folder stores the tensor under
+    store_name: Callable[[str], str] = field(default=lambda name: name)
     eos_token_id: Optional[int] = None

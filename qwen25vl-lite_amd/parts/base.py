@@ -83,6 +83,9 @@ class LayerSlot:
     v_cache: Optional[torch.Tensor] = None  # [pages, nkv, hd, page_size]
     writes: bool = True
     state: Optional[torch.Tensor] = None    # [max_num_seqs, *StateNeed.shape]
+    # a block with several mixers: each one's slot under the mixer's sub-part name (this slot is
+    # the first of them)
+    by_part: Dict[str, "LayerSlot"] = field(default_factory=dict)
 
 
 @dataclass

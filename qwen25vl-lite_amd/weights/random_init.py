@@ -16,7 +16,7 @@ from typing import Dict, Iterator, Optional, Tuple
 
 import torch
 
-from ..config.model_config import Qwen25VLConfig
+from ..config.registry import config_to_dict
 from .safetensors_io import write_safetensors
 
 __all__ = ["random_tensors", "write_random_model", "fill_random"]
@@ -49,22 +49,26 @@ def random_tensors(model, seed: int, std: float = 0.02, *, device="cpu",
         yield name, _draw(name, spec.shape, seed, std, device, dtype or torch.float32, spec.role)
 
 
-def write_random_model(config: Qwen25VLConfig, out_dir: str, seed: int, *, std: float = 0.02,
-                       dtype: torch.dtype = torch.bfloat16, prefix: str = "model.language_model.") -> str:
+def write_random_model(config, out_dir: str, seed: int, *, std: float = 0.02,
+                       dtype: torch.dtype = torch.bfloat16) -> str:
     """Write a model folder (``config.json``, ``model.safetensors``) with random weights.
 
-    Tensors are stored in ``dtype`` under the released checkpoints' names
-    (``model.language_model.layers...``, ``lm_head.weight``)."""
+    ``config`` is a configuration object of any registered architecture (or the dictionary of
+    its ``config.json``).  Tensors are stored in ``dtype`` under the names the architecture's
+    spec gives them in a checkpoint (for the Qwen2.5-VL decoder the released checkpoints'
+    ``model.language_model.layers...``, ``lm_head.weight``)."""
+    from ..config.registry import load_config
     from ..models import build_model
 
     os.makedirs(out_dir, exist_ok=True)
+    if isinstance(config, dict):
+        config = load_config(config)
     model = build_model(config, torch.float32, "meta")
     tensors: Dict[str, torch.Tensor] = {}
     for name, t in random_tensors(model, seed, std, dtype=dtype):
-        stored = name if name.startswith("lm_head.") else prefix + name
-        tensors[stored] = t
+        tensors[model.spec.store_name(name)] = t
     with open(os.path.join(out_dir, "config.json"), "w", encoding="utf-8") as fh:
-        json.dump(config.to_dict(), fh, indent=1)
+        json.dump(config_to_dict(config), fh, indent=1)
     write_safetensors(os.path.join(out_dir, "model.safetensors"), tensors)
     return out_dir
 

@@ -287,9 +287,9 @@ def test_everything_at_once(model_dirs, name, seed):
     assert llm.runner.cache.pages_in_use()[0] == cached
 
 
-@pytest.mark.parametrize("name, seed, pool, seqs", [("A", 3, 14, 5), ("C", 6, 20, 3)])
+@pytest.mark.parametrize("name, seed, pool, seqs", [("A", 3, 12, 5), ("C", 6, 14, 4)])
 def test_look_ahead_under_preemption_stops_arrivals_and_the_prefix_cache(model_dirs, name, seed, pool, seqs):
-    """The decode step queued ahead, in a server's day: requests arriving over forty steps, a shared
+    """The decode step queued ahead, in a server's day: requests arriving over a dozen steps, a shared
     prefix and the prefix cache (model A) or a windowed group (model C), stop tokens frequent enough
     to end some requests early (found out one step late), seeded sampling beside greedy, a request
     with a penalty, and so few pages that requests are preempted and computed again.  Tokens and
@@ -306,15 +306,13 @@ def test_look_ahead_under_preemption_stops_arrivals_and_the_prefix_cache(model_d
     prompts = [random_tokens(rng.randint(2, 50), vocab, 5000 + 50 * seed + i) for i in range(n)]
     for i in (0, 4, 7):
         prompts[i] = shared + prompts[i][:12]
-    stop_pool = tuple(rng.randrange(vocab) for _ in range(12))
     params = []
     for i in range(n):
         kind = rng.random()
         params.append(SamplingParams(temperature=0.0 if kind < 0.6 else 0.9, top_k=0 if kind < 0.8 else 30,
-                                     seed=rng.randint(0, 99), max_tokens=rng.randint(2, 50), ignore_eos=True,
-                                     stop_token_ids=stop_pool if i % 2 else (),
+                                     seed=rng.randint(0, 99), max_tokens=rng.randint(25, 60), ignore_eos=True,
                                      repetition_penalty=1.2 if i == 5 else 1.0))
-    arrive = sorted(rng.randint(0, 40) for _ in range(n))
+    arrive = sorted(rng.randint(0, 12) for _ in range(n))
     arrive[0] = 0
 
     def run(look):
@@ -336,6 +334,10 @@ def test_look_ahead_under_preemption_stops_arrivals_and_the_prefix_cache(model_d
         assert cache.pages_in_use()[0] == cached and all(u == 0 for u in cache.pages_in_use()[1:])
         return sorted(((o.seq_id, o.output_token_ids, o.finish_reason) for o in outs)), queued, eng.stats()
 
+    free, _, _ = run(False)
+    for sid, tokens, _ in free:        # every other request stops on a token it really produces, half way
+        if sid % 2 and len(tokens) >= 4:
+            params[sid].stop_token_ids = (tokens[len(tokens) // 2],)
     plain, none_queued, stats0 = run(False)
     ahead, queued, stats1 = run(True)
     assert none_queued == 0 and queued > 10, queued
@@ -497,6 +499,30 @@ def test_trace_run_program(model_dirs, tmp_path):
     s2 = torch.from_numpy(np.fromfile(out / "2.f32", dtype="<f4").reshape(2, 256))
     assert torch.allclose(s0, ref[[0, 8]], atol=1e-4, rtol=1e-3)
     assert torch.allclose(s2[0], ref[20], atol=1e-4, rtol=1e-3) and torch.allclose(s2[1], ref[2], atol=1e-4, rtol=1e-3)
+
+
+def test_generate_and_bench_commands(model_dirs):
+    """`qwen25vl-lite generate` as a user calls it (reference cli.py:267-278): two prompts separated
+    by ';', decode steps from a captured graph with the next step queued ahead; it prints each
+    request's list of output ids, which are the plain implementation's.  Without prompt ids it
+    exits with 2 (reference cli.py:271-274).  `bench` runs its one prompt and prints its rates."""
+    import ast
+    d = model_dirs["B_sharp"]
+    prompts = [[7, 300, 41, 2, 99], [5, 6]]
+    cli = [sys.executable, os.path.join(ROOT, "bin", "qwen25vl-lite")]
+    common = ["--model", d, "--dtype", "float32", "--num-blocks", "32", "--max-num-seqs", "2", "--max-model-len", "256"]
+    proc = subprocess.run(cli + ["generate", *common, "--cuda-graph", "--decode-lookahead", "--max-tokens", "9",
+                                 "--ignore-eos", "--prompt-token-ids", ";".join(",".join(map(str, p)) for p in prompts)],
+                          capture_output=True, text=True, timeout=110)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    printed = [ast.literal_eval(line) for line in proc.stdout.strip().splitlines()]
+    assert printed == [_plain_greedy(d, p, 9) for p in prompts]
+    proc = subprocess.run(cli + ["generate", *common], capture_output=True, text=True, timeout=110)
+    assert proc.returncode == 2 and "--prompt-token-ids" in proc.stderr
+    proc = subprocess.run(cli + ["bench", *common, "--prompt-tokens", "40", "--max-tokens", "6"],
+                          capture_output=True, text=True, timeout=110)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert "prefill 40 tokens + decode 6 tokens" in proc.stdout and "tok/s" in proc.stdout
 
 
 def test_smoke_entry():

@@ -319,3 +319,168 @@ def test_toy_parts_register_build_and_step():
     # a slot that is taken again starts from a cleared state
     runner.release("a"); runner.release("b")
     assert torch.allclose(_run(runner, "again", tb, [21]), want_b, atol=2e-4)
+
+
+# ---------------------------------------------------------------------------------------------
+# a whole toy architecture, from a model folder, with nothing but registrations
+# ---------------------------------------------------------------------------------------------
+TOY_CONFIG = {
+    "architectures": ["ToyDecayLM"], "width": 24, "tokens": 40, "state": 10, "inner": 40, "heads": 3, "groups": 1,
+    "head": 8, "reach": 9, "base": 50.0, "stop_id": 39,
+    # which mixer and feed-forward each layer has; no key of the Qwen decoder appears anywhere
+    "plan": [["decay", "routed"], ["attention", "swiglu"], ["decay", "swiglu"]],
+}
+
+
+def _register_toy_architecture():
+    from qwen25vl_lite_amd.config import known_architectures, register_architecture
+    from qwen25vl_lite_amd.models import LayerSpec, ModelSpec, RunEntry
+    from qwen25vl_lite_amd.parts import PartSpec
+    _register_toys()
+    if "ToyDecayLM" in known_architectures():
+        return
+
+    def build_spec(cfg):
+        hidden = cfg.width
+        norm = PartSpec("rms_norm", {"size": hidden, "eps": 1e-6})
+        pos = PartSpec("toy_half_speed", {"theta": cfg.base})
+        mixers = {"decay": PartSpec("toy_decay", {"hidden_size": hidden, "state_size": cfg.state}),
+                  "attention": _attn_spec(hidden, cfg.heads, cfg.groups, cfg.head, pos, window=cfg.reach)}
+        ffns = {"routed": PartSpec("toy_routed", {"hidden_size": hidden}),
+                "swiglu": PartSpec("swiglu", {"hidden_size": hidden, "intermediate_size": cfg.inner})}
+        layers = []
+        for i, (mixer, ffn) in enumerate(cfg.plan):
+            block = PartSpec("pre_norm", {"norm1": norm, "mixer": mixers[mixer], "norm2": norm, "ffn": ffns[ffn],
+                                          "names": {"norm1": "ln1", "mixer": "mix", "norm2": "ln2", "ffn": "ff"}})
+            layers.append(LayerSpec(block, f"blocks.{i}."))
+        return ModelSpec(hidden_size=hidden, vocab_size=cfg.tokens, layers=layers,
+                         run=[RunEntry(i) for i in range(len(layers))], final_norm=norm, tie_word_embeddings=True,
+                         position_rows=3, embed_name="tok.weight", final_norm_prefix="ln_f.",
+                         store_name=lambda name: "toy." + name,
+                         map_name=lambda name: name[4:] if name.startswith("toy.") else name,
+                         eos_token_id=cfg.stop_id)
+
+    register_architecture("ToyDecayLM", build_spec)      # no reader of its own: the raw keys are its configuration
+
+
+def test_toy_architecture_from_a_model_folder(tmp_path):
+    """A model folder whose config.json names an architecture registered here, with keys of its
+    own (none of the Qwen decoder's), a mixer with per-request state, a routed feed-forward and its
+    own position encoding: written with random weights, loaded through ``LLM``, replayed through
+    ``Replayer``, generated from greedily, with nothing but ``register_part`` and
+    ``register_architecture`` calls.  The prefix cache switches itself off (a cached prefix could
+    not bring the mixer's state back)."""
+    import json
+    from qwen25vl_lite_amd import LLM, SamplingParams, write_random_model
+    from qwen25vl_lite_amd.config import load_config
+    from qwen25vl_lite_amd.engine.replay import Replayer
+    from qwen25vl_lite_amd.weights import SafetensorsFile
+    _register_toy_architecture()
+    d = str(tmp_path / "toy")
+    write_random_model(load_config(TOY_CONFIG), d, seed=11, std=0.3, dtype=torch.float32)
+    with open(f"{d}/config.json") as fh:
+        assert json.load(fh) == TOY_CONFIG
+    with SafetensorsFile(f"{d}/model.safetensors") as f:
+        assert "toy.blocks.0.mix.B.weight" in f.keys() and "toy.tok.weight" in f.keys()
+    llm = LLM(d, dtype="float32", num_blocks=16, block_size=16, max_num_seqs=3, max_num_batched_tokens=16,
+              enable_prefix_cache=True)
+    assert llm.runner.cache.prefix_cache is None, "a model with per-request state must not reuse cached prefixes"
+    assert llm.runner.eos_token_id == 39
+    g = torch.Generator().manual_seed(4)
+    prompts = [torch.randint(0, 39, (n,), generator=g).tolist() for n in (5, 23, 12)]
+    # the second shares the first's opening tokens: with a prefix cache it would skip them
+    prompts[1][:5] = prompts[0]
+    outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=7, ignore_eos=True))
+    for prompt, out in zip(prompts, outs):
+        ids, want = list(prompt), []
+        for _ in range(7):
+            nxt = int(torch.argmax(_plain_toy_model(llm.model, ids, torch.arange(len(ids)))[-1]))
+            want.append(nxt)
+            ids.append(nxt)
+        assert out.output_token_ids == want
+    assert llm.engine.stats()["prefix_cache_hits"] == 0
+    # the same folder through the replay tool's class: whole, then cut
+    rp = Replayer(d, "float32", 64)
+    toks = prompts[1]
+    whole = rp.step({"step": 0, "entries": [{"id": "w", "tokens": toks, "want": list(range(len(toks)))}], "end": ["w"]})
+    want = _plain_toy_model(llm.model, toks, torch.arange(len(toks)))
+    assert torch.allclose(whole.cpu(), want, atol=2e-4)
+    rows = []
+    for i, (a, b) in enumerate(((0, 9), (9, 11), (11, 23))):
+        rows.append(rp.step({"step": i + 1, "entries": [{"id": "c", "tokens": toks[a:b], "want": list(range(b - a))}]}))
+    assert torch.allclose(torch.cat(rows).cpu(), want, atol=2e-4)
+
+
+def test_a_block_with_two_mixers_gets_a_slot_for_each():
+    """A block defined here runs an attention mixer and a state mixer side by side on the same
+    normalised input.  The model gives each its own place: pages for one, a state row for the
+    other, found under the mixer's sub-part name.  Whole, cut and interleaved runs agree, and
+    both mixers contribute."""
+    from qwen25vl_lite_amd.engine import StepEntry
+    from qwen25vl_lite_amd.models import DecoderModel, LayerSpec, ModelSpec, RunEntry
+    from qwen25vl_lite_amd.parts import Block, PartSpec, build_part, known_parts, register_part
+    from qwen25vl_lite_amd.weights import fill_random
+    _register_toys()
+
+    class SideBySide(Block):
+        def __init__(self, params, dtype, device):
+            super().__init__(dtype, device)
+            self.norm1 = build_part("norm", params["norm"], dtype, device)
+            self.attn = build_part("mixer", params["attn"], dtype, device)
+            self.decay = build_part("mixer", params["decay"], dtype, device)
+            self.norm2 = build_part("norm", params["norm"], dtype, device)
+            self.ffn = build_part("ffn", params["ffn"], dtype, device)
+
+        def sub_parts(self):
+            return {"ln1": self.norm1, "attn": self.attn, "decay": self.decay, "ln2": self.norm2, "ff": self.ffn}
+
+        def forward(self, stream, step, slot):
+            x = self.norm1.forward(stream)
+            a = self.attn.forward(x, step, slot.by_part["attn"])
+            b = self.decay.forward(x, step, slot.by_part["decay"])
+            stream.pending = a.float() + b
+            y = self.norm2.forward(stream)
+            stream.pending = self.ffn.forward(y, step)
+            return stream
+
+    if "toy_side_by_side" not in known_parts("block"):
+        register_part("block", "toy_side_by_side", SideBySide)
+    hidden = 24
+    norm = PartSpec("rms_norm", {"size": hidden, "eps": 1e-6})
+    pos = PartSpec("rope", {"theta": 100.0, "rotary_dim": 8})
+    block = PartSpec("toy_side_by_side", {
+        "norm": norm, "attn": _attn_spec(hidden, 3, 1, 8, pos), "ffn": PartSpec("toy_routed", {"hidden_size": hidden}),
+        "decay": PartSpec("toy_decay", {"hidden_size": hidden, "state_size": 6})})
+    spec = ModelSpec(hidden_size=hidden, vocab_size=40, layers=[LayerSpec(block, "b0."), LayerSpec(block, "b1.")],
+                     run=[RunEntry(0), RunEntry(1)], final_norm=norm, tie_word_embeddings=True, position_rows=3,
+                     embed_name="tok.weight", final_norm_prefix="ln_f.")
+    model = DecoderModel(spec, torch.float32, "cuda:0")
+    fill_random(model, 8, std=0.3)
+    assert model.entry_places == [{"attn": 0, "decay": 1}, {"attn": 2, "decay": 3}]
+    assert [s is not None for s in model.entry_state] == [False, True, False, True]
+    assert model.cache_groups()[0].num_layers == 2
+    runner = _runner(model, pages=8)
+    slot = runner.slots[1]
+    assert slot.by_part["attn"].k_cache is not None and slot.by_part["attn"].state is None
+    assert slot.by_part["decay"].k_cache is None and slot.by_part["decay"].state.shape == (5, 6)
+    g = torch.Generator().manual_seed(2)
+    ta = torch.randint(0, 40, (26,), generator=g).tolist()
+    tb = torch.randint(0, 40, (9,), generator=g).tolist()
+    whole_a, whole_b = _run(runner, "a", ta, [26]), _run(runner, "b", tb, [9])
+    assert torch.allclose(_run(runner, "a2", ta, [3, 2, 17, 1, 1, 2]), whole_a, atol=1e-5)
+    runner.admit("a"); runner.admit("b")
+    got_a, got_b = [], []
+    for i in range(9):                       # portions of a beside single tokens of b
+        n = 3 if i < 8 else 2
+        out = runner.execute([StepEntry("b", tb[i:i + 1], i, want=[0]),
+                              StepEntry("a", ta[3 * i:3 * i + n], 3 * i, want=list(range(n)))]).cpu()
+        got_b.append(out[:1]); got_a.append(out[1:])
+    assert torch.allclose(torch.cat(got_a), whole_a, atol=1e-5) and torch.allclose(torch.cat(got_b), whole_b, atol=1e-5)
+    runner.release("a"); runner.release("b")
+    # each mixer matters: without its output projection the logits change
+    for name in ("b0.attn.o_proj.weight", "b1.decay.C.weight"):
+        part, local, _ = model.params[name]
+        kept = (part.w_out if local == "o_proj.weight" else part.C).clone()
+        (part.w_out if local == "o_proj.weight" else part.C).zero_()
+        assert not torch.allclose(_run(runner, "z", ta, [26]), whole_a, atol=1e-3)
+        (part.w_out if local == "o_proj.weight" else part.C).copy_(kept)
