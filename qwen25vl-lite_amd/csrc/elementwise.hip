@@ -34,7 +34,9 @@ extern "C" int qvl_embed_gather(const void* ids, const void* table, void* out, i
 
 // ---------------------------------------------------------------------------------------
 // Residual add + RMSNorm  (reference layers.py:27-31, text.py:196-205)
-//   v = h[row] + delta[row]            (delta optional; the sum is float32)
+//   v = h[row] + delta[row]            (delta optional; the sum is float32; delta may come as
+//                                       several slabs [slab][row], partial sums of a product cut
+//                                       along its inner size, which are added in slab order)
 //   h[row] = v                         (unless `rows` selects rows: then h is left alone)
 //   out[m] = v * (1/sqrt(mean(v^2) + eps)) * w
 // One block per row; the reduction order depends on H only, so a row's result does not
@@ -42,16 +44,22 @@ extern "C" int qvl_embed_gather(const void* ids, const void* table, void* out, i
 // ---------------------------------------------------------------------------------------
 template <typename TD, typename TO>
 __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__ delta, const float* __restrict__ w,
-                                   TO* __restrict__ out, const int* __restrict__ rows, int H, float eps) {
+                                   TO* __restrict__ out, const int* __restrict__ rows, int H, float eps, int nslabs,
+                                   long long slab_stride) {
   __shared__ float red[17];
   const int m = blockIdx.x;
   const int row = rows ? rows[m] : m;
   float* hr = h + (size_t)row * H;
   const TD* dr = delta ? delta + (size_t)row * H : nullptr;
+  auto delta_at = [&](int i) {
+    float d = ldf<TD>(dr + i);
+    for (int c = 1; c < nslabs; ++c) d += ldf<TD>(dr + (size_t)c * slab_stride + i);
+    return d;
+  };
   float ss = 0.f;
   for (int i = threadIdx.x; i < H; i += blockDim.x) {
     float v = hr[i];
-    if (dr) v += ldf<TD>(dr + i);
+    if (dr) v += delta_at(i);
     ss += v * v;
     if (dr && !rows) hr[i] = v;
   }
@@ -60,7 +68,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__
   TO* o = out + (size_t)m * H;
   for (int i = threadIdx.x; i < H; i += blockDim.x) {
     float v = hr[i];
-    if (dr && rows) v += ldf<TD>(dr + i);
+    if (dr && rows) v += delta_at(i);
     stf<TO>(o + i, (v * rs) * w[i]);
   }
 }
@@ -88,7 +96,8 @@ template <> __device__ __forceinline__ void st4<bf16_t>(bf16_t* p, float4 v) {
 template <typename TD, typename TO>
 __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict__ h, const TD* __restrict__ delta,
                                                               const float* __restrict__ w, TO* __restrict__ out,
-                                                              const int* __restrict__ rows, int H, float eps) {
+                                                              const int* __restrict__ rows, int H, float eps,
+                                                              int nslabs, long long slab_stride) {
   __shared__ float red[17];
   const int m = blockIdx.x;
   const int row = rows ? rows[m] : m;
@@ -103,7 +112,11 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
     if (i < nvec) {
       float4 x = ld4<float>(hr + 4 * i);
       if (dr) {
-        const float4 d = ld4<TD>(dr + 4 * i);
+        float4 d = ld4<TD>(dr + 4 * i);
+        for (int c = 1; c < nslabs; ++c) {
+          const float4 e = ld4<TD>(dr + (size_t)c * slab_stride + 4 * i);
+          d.x += e.x; d.y += e.y; d.z += e.z; d.w += e.w;
+        }
         x.x += d.x; x.y += d.y; x.z += d.z; x.w += d.w;
         if (!rows) st4<float>(hr + 4 * i, x);
       }
@@ -123,20 +136,24 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
   }
 }
 
+// delta: null, or nslabs slabs of [rows of h][H], slab_stride elements apart (nslabs 1: one addend).
 extern "C" int qvl_add_rmsnorm(void* h, const void* delta, const void* w, void* out, const void* rows, int M, int H,
-                               float eps, int delta_dtype, int out_dtype, hipStream_t stream) {
+                               float eps, int delta_dtype, int out_dtype, int nslabs, long long slab_stride,
+                               hipStream_t stream) {
   if (M <= 0) return QVL_OK;
-  if (H <= 0) return QVL_ERR_SHAPE;
+  if (H <= 0 || nslabs < 1 || (nslabs > 1 && (slab_stride < H || slab_stride % 4))) return QVL_ERR_SHAPE;
   const int threads = H >= 2048 ? 512 : 256;
   const bool vec = H % 4 == 0 && H <= NORM_VEC_MAX * 4 * 256;
 #define QVL_NORM_CASE(DD, OD, TD, TO)                                                                              \
   if (delta_dtype == DD && out_dtype == OD) {                                                                      \
     if (vec)                                                                                                       \
       hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TO>), dim3(M), dim3(256), 0, stream, (float*)h,               \
-                         (const TD*)delta, (const float*)w, (TO*)out, (const int*)rows, H, eps);                   \
+                         (const TD*)delta, (const float*)w, (TO*)out, (const int*)rows, H, eps, nslabs,            \
+                         slab_stride);                                                                             \
     else                                                                                                           \
       hipLaunchKernelGGL((add_rmsnorm_kernel<TD, TO>), dim3(M), dim3(threads), 0, stream, (float*)h,               \
-                         (const TD*)delta, (const float*)w, (TO*)out, (const int*)rows, H, eps);                   \
+                         (const TD*)delta, (const float*)w, (TO*)out, (const int*)rows, H, eps, nslabs,            \
+                         slab_stride);                                                                             \
     return qvl_launch_status();                                                                                    \
   }
   QVL_NORM_CASE(0, 0, float, float)

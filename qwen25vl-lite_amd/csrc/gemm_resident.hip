@@ -1,4 +1,4 @@
-// Products with at most 32 rows (a decode step's projections): out[M, N] = X[M, K] . W[N, K]^T,
+// Products with at most 64 rows (a decode step's projections): out[M, N] = X[M, K] . W[N, K]^T,
 // bfloat16 operands, float32 accumulation.  The step is bound by reading W once from HBM, so W
 // is the streamed operand and everything around the product is folded into this kernel, because
 // between two products a short kernel of its own costs more than its arithmetic (its code and
@@ -11,7 +11,10 @@
 // Wave w covers the 256 values of K from 256 w on, as the A operand (W rows) and B operand (X
 // rows) of v_mfma_f32_16x16x32_bf16; the 16 waves' sums meet in LDS and are added in wave order.
 // Up to 16 rows of X are one column tile of the matrix instruction; 17 to 32 rows are two (MT = 2):
-// every W fragment that is loaded is multiplied with both.
+// every W fragment that is loaded is multiplied with both.  33 to 64 rows are four (MT = 4): they
+// fit neither the registers nor LDS, so X is not resident: for every tile of W each wave reads its
+// columns of all rows of X again (from L2: four times the bytes of the tile's W), and a norm is
+// not folded in (the host hands over normalised rows).
 // If K fits one pass (K <= 4096) the X operand stays in registers (the second column tile, if
 // there is one, in LDS, which takes K <= 32 * XHI_STEPS) for all of the block's tiles; W comes
 // through three half-tile buffers that go round, so that the next tile and a half are on their way
@@ -57,6 +60,11 @@ struct ResidentArgs {
   int ldo;
   int M, N, K, ntiles;
   int rows;              // rows of W per tile, 1..16 (16 with EPI_SWIGLU and EPI_ROPE)
+  // More rows of X than a block carries: `groups` blocks form a team that walks the same tiles of W,
+  // block g of the team with rows g * (16 MT) ... of X.  The blocks of a team run on the same XCD
+  // at the same pace, so the tile that the first of them brings in from HBM the others find in
+  // that XCD's L2 (or in the memory-side cache): W leaves HBM once.
+  int groups;
   // EPI_ROPE: W rows are nq query heads, nkv key heads, nkv value heads of hd channels each
   // (hd a multiple of 16, rotation over the whole head in pairs (f, f + hd/2))
   const float* cs;       // [M, hd/2, 2] cosine and sine of each token's angle at each frequency
@@ -89,6 +97,8 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
   constexpr int COLS = 16 * MT;   // rows of X the block carries
   // MT = 1: two buffers, a tile's sums are read while the next tile's are written.  MT = 2: one
   // (LDS also holds the second column tile of X), and the norm weights borrow it before the first tile.
+  static_assert(MT == 1 || MT == 2 || MT == 4, "one, two or four column tiles");
+  static_assert(MT != 4 || PRO == PRO_PLAIN, "with four column tiles the rows arrive normalised");
   __shared__ __attribute__((aligned(16))) float red[MT == 1 ? 2 : 1][RW][16 * COLS];
   __shared__ float rowsq[RW][16];
   __shared__ __attribute__((aligned(16))) float gains_own[(PRO == PRO_NORM && MT == 1) ? RW : 1][RK * 32];
@@ -96,13 +106,22 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
   float (*gains)[RK * 32] = MT == 1 ? gains_own : reinterpret_cast<float (*)[RK * 32]>(&red[0][0][0]);  // norm weights of each wave's columns
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, lg = lane >> 4, r = lane & 15;
   const int k_lane = wave * RK * 32 + 8 * lg;  // first K index of this lane within a pass
+  // Workgroups go to the XCDs in turn, so blocks b, b + 8, b + 16, ... share an XCD: consecutive
+  // ones of them form a team.
+  int team = blockIdx.x, teams = gridDim.x, m0 = 0;   // m0: this block's first row of X
+  if (p.groups > 1) {   // the grid is a multiple of 8 groups
+    const int xcd_turn = blockIdx.x >> 3;
+    team = (xcd_turn / p.groups) * 8 + (blockIdx.x & 7);
+    teams = (int)(gridDim.x >> 3) / p.groups * 8;
+    m0 = (xcd_turn % p.groups) * COLS;
+  }
 
   // ---- the X operand of one pass ------------------------------------------------------------
   // Column tile t holds rows 16 t .. 16 t + 15 of X.  first_w issues the block's first W loads at
   // the point of the prologue where they fit best.  again: another column tile's norm came before
   // (the norm weights are in LDS already, and the statistics' place may still be read).
   auto load_x = [&](int t, int k0, bf16x8_t* xb, auto first_w, bool again = false) {
-    const int row = 16 * t + r;
+    const int row = m0 + 16 * t + r;
     const bool m_ok = row < p.M;
     if (PRO == PRO_PLAIN) {
       first_w();   // W first: it is the long wait
@@ -209,7 +228,7 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
     e.cs = float2{1.f, 0.f};
     e.slot = -1;
     if (threadIdx.x >= 16 * COLS || EPI == EPI_SWIGLU) return e;
-    const int m = threadIdx.x >> 4, nl = threadIdx.x & 15, n = w_row(tile, nl);
+    const int m = m0 + (threadIdx.x >> 4), nl = threadIdx.x & 15, n = w_row(tile, nl);
     if (m >= p.M || nl >= tile_rows(tile) || n >= p.N) return e;
     if (p.bias) e.bias = p.bias[n];
     if (EPI == EPI_RESIDUAL) e.old = reinterpret_cast<const float*>(p.out)[(size_t)m * p.ldo + n];
@@ -239,7 +258,7 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
     __syncthreads();
     if (threadIdx.x < 16 * COLS) {
       const int e = threadIdx.x;
-      const int m = e >> 4, nl = e & 15, n = w_row(tile, nl);
+      const int m = m0 + (e >> 4), nl = e & 15, n = w_row(tile, nl);
       float sum = 0.f;
 #pragma unroll
       for (int w = 0; w < RW; ++w) sum += buf[w][e];
@@ -277,23 +296,72 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
         }
       }
     }
-    if (MT == 2) __syncthreads();
+    if (MT >= 2) __syncthreads();
   };
   // The W operand's steps come as two halves (a_lo, a_hi).  x1: the second column tile's operand in
   // registers; null: it is in LDS (one pass), except for the waves whose steps lie beyond K then.
   const bool hi_live = wave * RK < XHI_STEPS;
-  auto product = [&](const bf16x8_t* a_lo, const bf16x8_t* a_hi, const bf16x8_t* x0, const bf16x8_t* x1, Acc acc) {
+  // steps u0 .. u0 + n - 1 of a tile, whose W operands are a[0 .. n - 1]
+  auto product_part = [&](const bf16x8_t* a, int u0, int n, const bf16x8_t* x0, const bf16x8_t* x1, Acc acc) {
 #pragma unroll
-    for (int u = 0; u < RK; ++u) {
-      const bf16x8_t a = u < RK / 2 ? a_lo[u] : a_hi[u - RK / 2];
-      acc.t[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, x0[u], acc.t[0], 0, 0, 0);
+    for (int i = 0; i < n; ++i) {
+      const int u = u0 + i;
+      acc.t[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], x0[u], acc.t[0], 0, 0, 0);
       if (MT == 2) {
         if (!ONE_PASS)
-          acc.t[MT - 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, x1[u], acc.t[MT - 1], 0, 0, 0);
+          acc.t[MT - 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], x1[u], acc.t[MT - 1], 0, 0, 0);
         else if (hi_live)
           acc.t[MT - 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-              a, __builtin_bit_cast(bf16x8_t, xhi[(wave * RK + u) * 64 + lane]), acc.t[MT - 1], 0, 0, 0);
+              a[i], __builtin_bit_cast(bf16x8_t, xhi[(wave * RK + u) * 64 + lane]), acc.t[MT - 1], 0, 0, 0);
       }
+    }
+    return acc;
+  };
+  auto product = [&](const bf16x8_t* a_lo, const bf16x8_t* a_hi, const bf16x8_t* x0, const bf16x8_t* x1, Acc acc) {
+    acc = product_part(a_lo, 0, RK / 2, x0, x1, acc);
+    return product_part(a_hi, RK / 2, RK / 2, x0, x1, acc);
+  };
+  // half of the plain X operand of the pass that starts at k0 (column tile 0): steps half * RK / 2 ...
+  auto load_x_half = [&](int k0, int half, bf16x8_t* xb) {
+    const int row = m0 + r;
+    const bool m_ok = row < p.M;
+    const bf16_t* xrow = p.X + (size_t)(m_ok ? row : 0) * p.ldx;
+#pragma unroll
+    for (int i = 0; i < RK / 2; ++i) {
+      const int u = half * (RK / 2) + i, k = k0 + k_lane + u * 32;
+      xb[u] = (m_ok && k < p.K) ? load8(xrow + k) : zero8();
+    }
+  };
+  // MT = 4: the X operands of the pass that starts at k0 come from memory (L2) for every tile, two
+  // steps of a column tile at a time through two small buffers that take turns, so that the next
+  // loads are on their way while these are multiplied (and the other waves of the SIMD fill the rest
+  // of the wait).
+  auto product_streamed = [&](const bf16x8_t* a_lo, const bf16x8_t* a_hi, int k0, Acc acc) {
+    constexpr int Q = 2, PARTS = RK / Q, CHUNKS = MT * PARTS;
+    bf16x8_t xs[2][Q];
+    auto load_chunk = [&](int c, bf16x8_t* dst) {
+      const int t = c / PARTS, part = c % PARTS;
+      const int row = m0 + 16 * t + r;
+      const bool m_ok = row < p.M;
+      const bf16_t* xrow = p.X + (size_t)(m_ok ? row : 0) * p.ldx;
+#pragma unroll
+      for (int u = 0; u < Q; ++u) {
+        const int k = k0 + k_lane + (part * Q + u) * 32;
+        dst[u] = (m_ok && k < p.K) ? load8(xrow + k) : zero8();
+      }
+    };
+    load_chunk(0, xs[0]);
+    load_chunk(1, xs[1]);
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+      const int t = c / PARTS, part = c % PARTS;
+#pragma unroll
+      for (int u = 0; u < Q; ++u) {
+        const int step = part * Q + u;
+        const bf16x8_t a = step < RK / 2 ? a_lo[step] : a_hi[step - RK / 2];
+        acc.t[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, xs[c & 1][u], acc.t[t], 0, 0, 0);
+      }
+      if (c + 2 < CHUNKS) load_chunk(c + 2, xs[c & 1]);
     }
     return acc;
   };
@@ -301,7 +369,7 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
 #pragma unroll
   for (int t = 0; t < MT; ++t) zero.t[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-  if (ONE_PASS || MT == 1) {
+  if (ONE_PASS || MT == 1 || MT == 4) {
     // The block's work is a sequence of steps: every tile of its own, and within a tile every pass
     // over K (one, if X stays resident).  Three half-step buffers of W go round: while a step is
     // multiplied, the first half of the next is on its way; its second half and the first half of
@@ -311,13 +379,18 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
     auto step_after = [&](int& t, int& ps) {
       if (++ps >= passes) {
         ps = 0;
-        t += gridDim.x;
+        t += teams;
       }
     };
     bf16x8_t xb[RK];
     bf16x8_t w[3][RK / 2];
-    int tile = blockIdx.x, pass = 0;
-    if (MT == 1) {
+    int tile = team, pass = 0;
+    if (MT == 4) {
+      if (tile < p.ntiles) {
+        load_w_part(tile, 0, 0, RK / 2, w[0]);
+        load_w_part(tile, 0, RK / 2, RK / 2, w[1]);
+      }
+    } else if (MT == 1) {
       load_x(0, 0, xb, [&] {
         if (tile < p.ntiles) {
           load_w_part(tile, 0, 0, RK / 2, w[0]);
@@ -343,20 +416,33 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
     }
     Acc acc = zero;
     // one step whose halves are in a_lo and a_hi; false: it was the block's last
+    // A half buffer is asked for again the moment its steps are multiplied (not after the whole
+    // step): every half then has a whole period, a step and a merge, to arrive in.  Between the
+    // passes of a tile the next rows of X are asked for the same way, each half ahead of the W
+    // half that is needed with it (loads come back in the order they were asked for).
     auto one = [&](bf16x8_t* a_lo, bf16x8_t* a_hi) {
-      acc = product(a_lo, a_hi, xb, nullptr, acc);
       int tn = tile, pn = pass;
       step_after(tn, pn);
       int ta = tn, pa = pn;
       step_after(ta, pa);
       const bool tile_done = ONE_PASS || pn == 0;
       Epi e_next = e;
-      if (tile_done) e_next = epi_load(tn);
-      if (tn < p.ntiles) {
-        if (!ONE_PASS) load_x(0, pn * PASS_K, xb, [] {});
-        load_w_part(tn, pn * PASS_K, RK / 2, RK / 2, a_lo);
+      if constexpr (MT == 4) {
+        acc = product_streamed(a_lo, a_hi, pass * PASS_K, acc);
+        if (tile_done) e_next = epi_load(tn);
+        if (tn < p.ntiles) load_w_part(tn, pn * PASS_K, RK / 2, RK / 2, a_lo);
+        if (ta < p.ntiles) load_w_part(ta, pa * PASS_K, 0, RK / 2, a_hi);
+      } else {
+        acc = product_part(a_lo, 0, RK / 2, xb, nullptr, acc);
+        if (tn < p.ntiles) {
+          if (!ONE_PASS && MT == 1) load_x_half(pn * PASS_K, 0, xb);
+          load_w_part(tn, pn * PASS_K, RK / 2, RK / 2, a_lo);
+        }
+        acc = product_part(a_hi, RK / 2, RK / 2, xb, nullptr, acc);
+        if (tile_done) e_next = epi_load(tn);
+        if (tn < p.ntiles && !ONE_PASS && MT == 1) load_x_half(pn * PASS_K, 1, xb);
+        if (ta < p.ntiles) load_w_part(ta, pa * PASS_K, 0, RK / 2, a_hi);
       }
-      if (ta < p.ntiles) load_w_part(ta, pa * PASS_K, 0, RK / 2, a_hi);
       if (tile_done) {
         finish(tile, acc, e);
         acc = zero;
@@ -372,7 +458,7 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
       if (!one(w[1], w[2])) break;
     }
   } else {
-    for (int tile = blockIdx.x; tile < p.ntiles; tile += gridDim.x) {
+    for (int tile = team; tile < p.ntiles; tile += teams) {
       Acc acc = zero;
       const Epi e = epi_load(tile);
       for (int k0 = 0; k0 < p.K; k0 += PASS_K) {
@@ -386,19 +472,57 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
   }
 }
 
+// How M rows are carried: column tiles per block (MT), blocks per team (groups), and whether X stays
+// in the block for all its tiles (one pass over K).  Up to 32 rows one block carries them all.
+// More rows, or 17 to 32 rows with a K too long for the second column tile's place in LDS, are
+// spread over the blocks of a team; a device with too few compute units for teams (fewer than 8
+// per group) falls back on one block that streams X (MT = 4).
+struct Plan {
+  int mt, groups;
+  bool one_pass;
+};
+static Plan plan_for(int M, int K, bool norm, int blocks, bool prefer_teams) {
+  if (M <= 16) return Plan{1, 1, K <= PASS_K};
+  const bool two_fit = K <= 32 * XHI_STEPS;
+  if (M <= 32 && two_fit) return Plan{2, 1, true};
+  if (two_fit && blocks >= 8 * ((M + 31) / 32)) return Plan{2, (M + 31) / 32, true};
+  const int singles = (M + 15) / 16;
+  if ((M > 32 || prefer_teams || norm) && blocks >= 8 * singles) return Plan{1, singles, K <= PASS_K};
+  if (M <= 32) return Plan{2, 1, false};
+  return Plan{4, 1, K <= PASS_K};
+}
+// the number of teams the plan's grid has: what the tiles are divided among
+static int plan_teams(const Plan& pl, int blocks) { return pl.groups == 1 ? blocks : blocks / (8 * pl.groups) * 8; }
+
 template <typename TO, int PRO, int EPI>
-static void launch(const ResidentArgs& p, int blocks, hipStream_t stream) {
-  const dim3 grid(blocks < p.ntiles ? blocks : p.ntiles), block(64 * RW);
-  if (p.K <= PASS_K && p.M <= 16)
-    hipLaunchKernelGGL((gemm_resident_kernel<TO, PRO, EPI, true, 1>), grid, block, 0, stream, p);
-  else if (p.K <= 32 * XHI_STEPS)
-    hipLaunchKernelGGL((gemm_resident_kernel<TO, PRO, EPI, true, 2>), grid, block, 0, stream, p);
-  else if constexpr (PRO == PRO_PLAIN) {   // a norm is only folded into a single pass: the host has checked
-    if (p.M <= 16)
-      hipLaunchKernelGGL((gemm_resident_kernel<TO, PRO, EPI, false, 1>), grid, block, 0, stream, p);
-    else
-      hipLaunchKernelGGL((gemm_resident_kernel<TO, PRO, EPI, false, 2>), grid, block, 0, stream, p);
+static int launch(ResidentArgs p, const Plan& pl, int blocks, hipStream_t stream) {
+  const int teams = plan_teams(pl, blocks);
+  p.groups = pl.groups;
+  const dim3 grid(pl.groups == 1 ? (teams < p.ntiles ? teams : p.ntiles) : teams * pl.groups), block(64 * RW);
+#define QVL_GO(ONE, MT) hipLaunchKernelGGL((gemm_resident_kernel<TO, PRO, EPI, ONE, MT>), grid, block, 0, stream, p)
+  if (PRO == PRO_NORM && !pl.one_pass) return QVL_ERR_LIMIT;   // a norm is only folded into a single pass
+  if (pl.mt == 1) {
+    if (pl.one_pass) QVL_GO(true, 1);
+    else if constexpr (PRO == PRO_PLAIN) QVL_GO(false, 1);
+  } else if (pl.mt == 2) {
+    if (pl.one_pass) QVL_GO(true, 2);
+    else if constexpr (PRO == PRO_PLAIN) QVL_GO(false, 2);
+  } else if constexpr (PRO == PRO_PLAIN) {
+    if (pl.one_pass) QVL_GO(true, 4);
+    else QVL_GO(false, 4);
+  } else {
+    return QVL_ERR_LIMIT;
   }
+#undef QVL_GO
+  return qvl_launch_status();
+}
+
+// Whether qvl_gemm_resident(_rope) forms the norm of M rows of width K itself on a device with this
+// many compute units.
+extern "C" int qvl_gemm_resident_folds_norm(int M, int K, int blocks) {
+  if (M <= 0 || M > 64 || K <= 0 || K > PASS_K || blocks <= 0) return 0;
+  const Plan pl = plan_for(M, K, true, blocks, false);
+  return pl.one_pass && pl.mt <= 2;
 }
 
 extern "C" int qvl_gemm_resident_pass_k() { return PASS_K; }
@@ -411,14 +535,18 @@ extern "C" int qvl_gemm_resident_two_tile_k() { return 32 * XHI_STEPS; }
 // max_blocks: blocks to launch at most (the number of compute units).
 extern "C" int qvl_gemm_resident(const void* x, int ldx, const void* h, int ldh, const void* norm_w, float eps,
                                  const void* W, int ldw, const void* bias, void* out, int ldo, int M, int N, int K,
-                                 int out_dtype, int epilogue, int max_blocks, hipStream_t stream) {
+                                 int out_dtype, int epilogue, int max_blocks, int flags, hipStream_t stream) {
+  // flags bit 0: 17 to 32 rows with a long K go to a team of two blocks rather than to one block
+  // that reads its rows again for every pass
   if (M <= 0 || N <= 0) return QVL_OK;
-  if (M > 32) return QVL_ERR_LIMIT;
+  if (M > 64) return QVL_ERR_LIMIT;
   if (K <= 0 || K % 8 || ldw % 8 || ldw < K || max_blocks <= 0 || !W || !out) return QVL_ERR_SHAPE;
   const bool norm = h != nullptr;
+  const Plan pl = plan_for(M, K, norm, max_blocks, flags & 1);
+  const int teams = plan_teams(pl, max_blocks);
   if (norm) {
     if (x || !norm_w || K > PASS_K || ldh % 4 || ldh < K) return QVL_ERR_SHAPE;
-    if (M > 16 && K > 32 * XHI_STEPS) return QVL_ERR_LIMIT;
+    if (!qvl_gemm_resident_folds_norm(M, K, max_blocks)) return QVL_ERR_LIMIT;
   } else if (!x || ldx % 8 || ldx < K) {
     return QVL_ERR_SHAPE;
   }
@@ -436,33 +564,29 @@ extern "C" int qvl_gemm_resident(const void* x, int ldx, const void* h, int ldh,
   // as many rounds of tiles as 16-row tiles need, with rows per tile cut down to what fills them evenly
   p.rows = 16;
   if (epilogue != EPI_SWIGLU) {
-    const long long per_round = 16LL * max_blocks;
+    const long long per_round = 16LL * teams;
     const long long rounds = (N + per_round - 1) / per_round;
-    p.rows = (int)((N + rounds * max_blocks - 1) / (rounds * max_blocks));
+    p.rows = (int)((N + rounds * teams - 1) / (rounds * teams));
   }
   p.ntiles = (N + p.rows - 1) / p.rows;
   p.whole_tiles = p.ntiles; p.parts = 1; p.pairs = 8;
   if (epilogue == EPI_SWIGLU) {
-    const int groups = N / 16, left = groups % max_blocks;
-    if (groups > max_blocks && left > 0) {
-      while (p.parts < 8 && left * p.parts * 2 <= max_blocks) p.parts *= 2;
+    const int groups = N / 16, left = groups % teams;
+    if (groups > teams && left > 0) {
+      while (p.parts < 8 && left * p.parts * 2 <= teams) p.parts *= 2;
       p.pairs = 8 / p.parts;
       p.whole_tiles = groups - left;
       p.ntiles = p.whole_tiles + left * p.parts;
     }
   }
-#define QVL_RES(TO, EPI)                                                    \
-  do {                                                                      \
-    if (norm) launch<TO, PRO_NORM, EPI>(p, max_blocks, stream);             \
-    else launch<TO, PRO_PLAIN, EPI>(p, max_blocks, stream);                 \
-  } while (0)
+#define QVL_RES(TO, EPI) \
+  return norm ? launch<TO, PRO_NORM, EPI>(p, pl, max_blocks, stream) : launch<TO, PRO_PLAIN, EPI>(p, pl, max_blocks, stream)
   if (epilogue == EPI_STORE && out_dtype == 0) QVL_RES(float, EPI_STORE);
-  else if (epilogue == EPI_STORE && out_dtype == 1) QVL_RES(bf16_t, EPI_STORE);
-  else if (epilogue == EPI_RESIDUAL) QVL_RES(float, EPI_RESIDUAL);
-  else if (epilogue == EPI_SWIGLU) QVL_RES(bf16_t, EPI_SWIGLU);
-  else return QVL_ERR_DTYPE;
+  if (epilogue == EPI_STORE && out_dtype == 1) QVL_RES(bf16_t, EPI_STORE);
+  if (epilogue == EPI_RESIDUAL) QVL_RES(float, EPI_RESIDUAL);
+  if (epilogue == EPI_SWIGLU) QVL_RES(bf16_t, EPI_SWIGLU);
 #undef QVL_RES
-  return qvl_launch_status();
+  return QVL_ERR_DTYPE;
 }
 
 // The stacked query | key | value projection of at most 32 tokens with rotation and cache write
@@ -477,14 +601,16 @@ extern "C" int qvl_gemm_resident_rope(const void* x, int ldx, const void* h, int
                                       const void* slot, void* q_out, void* kc, void* vc, int nq, int nkv, int hd, int ps,
                                       int max_blocks, hipStream_t stream) {
   if (M <= 0) return QVL_OK;
-  if (M > 32) return QVL_ERR_LIMIT;
+  if (M > 64) return QVL_ERR_LIMIT;
   if (K <= 0 || K % 8 || ldw % 8 || ldw < K || max_blocks <= 0 || !W || !q_out) return QVL_ERR_SHAPE;
   if (nq <= 0 || nkv < 0 || hd <= 0 || hd % 16 || ps <= 0 || !cs) return QVL_ERR_SHAPE;
   if (nkv > 0 && (!slot || !kc || !vc)) return QVL_ERR_SHAPE;
   const bool norm = h != nullptr;
+  const Plan pl = plan_for(M, K, norm, max_blocks, false);
+  const int teams = plan_teams(pl, max_blocks);
   if (norm) {
     if (x || !norm_w || K > PASS_K || ldh % 4 || ldh < K) return QVL_ERR_SHAPE;
-    if (M > 16 && K > 32 * XHI_STEPS) return QVL_ERR_LIMIT;
+    if (!qvl_gemm_resident_folds_norm(M, K, max_blocks)) return QVL_ERR_LIMIT;
   } else if (!x || ldx % 8 || ldx < K) {
     return QVL_ERR_SHAPE;
   }
@@ -498,16 +624,15 @@ extern "C" int qvl_gemm_resident_rope(const void* x, int ldx, const void* h, int
   p.rows = 16;
   int value_tiles = 0;
   if (nkv > 0) {
-    const long long vrows = (long long)nkv * hd, per_round = 16LL * max_blocks;
+    const long long vrows = (long long)nkv * hd, per_round = 16LL * teams;
     const long long rounds = (vrows + per_round - 1) / per_round;
-    p.rows = (int)((vrows + rounds * max_blocks - 1) / (rounds * max_blocks));
+    p.rows = (int)((vrows + rounds * teams - 1) / (rounds * teams));
     value_tiles = (int)((vrows + p.rows - 1) / p.rows);
   }
   p.ntiles = p.pair_tiles + value_tiles;
   p.cs = (const float*)cs; p.slot = (const int*)slot; p.q_out = (bf16_t*)q_out; p.kc = (bf16_t*)kc;
   p.vc = (bf16_t*)vc; p.nq = nq; p.nkv = nkv; p.hd = hd; p.ps = ps;
   p.whole_tiles = 0; p.parts = 1; p.pairs = 8;
-  if (norm) launch<bf16_t, PRO_NORM, EPI_ROPE>(p, max_blocks, stream);
-  else launch<bf16_t, PRO_PLAIN, EPI_ROPE>(p, max_blocks, stream);
-  return qvl_launch_status();
+  return norm ? launch<bf16_t, PRO_NORM, EPI_ROPE>(p, pl, max_blocks, stream)
+              : launch<bf16_t, PRO_PLAIN, EPI_ROPE>(p, pl, max_blocks, stream);
 }

@@ -15,8 +15,8 @@ LIBRARIES = [
     ("attention_generic", {}),
     ("gemm_f32", {}),
     ("sample", {}),
-    ("gemm_skinny", {}),
     ("gemm_resident", {}),
+    ("gemm_chunked", {}),
     # the matrix-core attention is compiled per head size; these are the sizes the tests and the
     # benchmark use, any other multiple of 16 is compiled at its first use
     ("attention_mfma", {"HD": 128}),

@@ -102,13 +102,20 @@ def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Te
     """``h += delta`` (float32 sum) and return ``rmsnorm(h) * weight`` in ``out_dtype``.
 
     With ``rows`` (int32 row indices) only those rows are normalised and ``h`` is not written.
+    ``delta`` may be float32 ``[slabs, N, H]``: partial sums of a product that was cut along its
+    inner size, added in slab order.
     """
     _dev(h, delta, weight, rows, out)
     _need(h.dtype == torch.float32 and h.dim() == 2 and h.is_contiguous(), "h must be contiguous float32 [N, H]")
     n, width = h.shape
     _need(weight.dtype == torch.float32 and weight.shape == (width,) and weight.is_contiguous(),
           "norm weight must be float32 [H]")
-    if delta is not None:
+    nslabs, slab_stride = 1, 0
+    if delta is not None and delta.dim() == 3:
+        _need(delta.dtype == torch.float32 and tuple(delta.shape[1:]) == tuple(h.shape) and delta.is_contiguous()
+              and width % 4 == 0, "slabs of delta must be contiguous float32 [slabs, N, H] with H in steps of 4")
+        nslabs, slab_stride = delta.shape[0], n * width
+    elif delta is not None:
         _need(delta.shape == h.shape and delta.is_contiguous(), "delta must match h's shape")
     m = n
     if rows is not None:
@@ -118,10 +125,11 @@ def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Te
         out = torch.empty((m, width), dtype=out_dtype, device=h.device)
     _need(out.shape == (m, width) and out.dtype == out_dtype and out.is_contiguous(), "out must be [M, H]")
     fn = _fn("elementwise", "qvl_add_rmsnorm",
-             [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr])
+             [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int,
+              ctypes.c_longlong, _c_ptr])
     _check(fn(_ptr(h), _ptr(delta), _ptr(weight), _ptr(out), _ptr(rows), m, width, float(eps),
-              dtype_code(delta.dtype if delta is not None else out_dtype), dtype_code(out_dtype), _stream()),
-           "add_rmsnorm")
+              dtype_code(delta.dtype if delta is not None else out_dtype), dtype_code(out_dtype), nslabs, slab_stride,
+              _stream()), "add_rmsnorm")
     return out
 
 
@@ -143,9 +151,9 @@ def rope_kv_write(x: torch.Tensor, bias: Optional[torch.Tensor], positions: torc
     kernel then reads the cosines and sines instead of computing them for every head.
     """
     _dev(x, bias, positions, inv_freq, freq_row, slots, k_cache, v_cache, q_out)
-    n = x.shape[0]
     nq, nkv, hd = int(num_q_heads), int(num_kv_heads), int(head_dim)
     cols = (nq + 2 * nkv) * hd
+    n = x.shape[0]
     _need(x.dim() == 2 and x.shape[1] == cols and x.stride(1) == 1, "x must be [N, (nq + 2 nkv) hd]")
     odt = out_dtype or x.dtype
     rot_half = inv_freq.shape[0]

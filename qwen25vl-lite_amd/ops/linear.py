@@ -1,9 +1,9 @@
 """Matrix products of the step: ``x @ weight.T`` for ``weight`` as a Linear stores it.
 
 float32 runs through the hand-written FMA kernel (true 32-bit, fixed summation order).
-bfloat16 with few rows (a decode step) runs through the hand-written matrix-core kernels, which
-also fold the norm before a product, the residual add after it and the SwiGLU activation into
-themselves; with many rows the vendor library's product runs, which is also what the
+bfloat16 with up to 64 rows (a decode step) runs through the hand-written matrix-core kernel, which
+also folds the norm before a product, the residual add after it and the SwiGLU activation into
+itself; with more rows the vendor library's product runs, which is also what the
 reference's engine uses for its projections (reference src/qwen25vl_lite/text.py:61-66, 80-90).
 """
 
@@ -49,17 +49,17 @@ def linear(x: Union[torch.Tensor, NormedRows], weight: torch.Tensor, bias: Optio
     if not weight.is_cuda:
         raise kernels.KernelError("linear has no CPU path: its tensors must be on the GPU")
     if weight.dtype == torch.bfloat16:
-        if lazy and skinny.takes_resident(m, k, weight, norm=True):
+        few = m <= skinny.ONE_BLOCK_ROWS     # beyond, the library streams a plain product faster
+        if lazy and few and skinny.takes_resident(m, k, weight, norm=True):
             return skinny.resident_product(weight, h=x.h, norm_weight=x.weight, eps=x.eps, bias=bias,
                                            out_dtype=out_dtype or torch.bfloat16)
         if lazy:
             x = x.materialize()
         if x.dtype != torch.bfloat16:
             raise kernels.KernelError(f"linear: operands {x.dtype}/{weight.dtype} are not built")
-        if skinny.takes_resident(m, k, weight) and x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0:
+        if few and skinny.takes_resident(m, k, weight) and _aligned(x):
             return skinny.resident_product(weight, x=x, bias=bias, out_dtype=out_dtype or torch.bfloat16)
-        out = skinny.try_streaming(x, weight, bias, out_dtype)
-        return out if out is not None else _library(x, weight, bias, out_dtype)
+        return _library(x, weight, bias, out_dtype)
     if lazy:
         x = x.materialize()
     if not x.is_cuda:
@@ -69,19 +69,33 @@ def linear(x: Union[torch.Tensor, NormedRows], weight: torch.Tensor, bias: Optio
     raise kernels.KernelError(f"linear: operands {x.dtype}/{weight.dtype} are not built")
 
 
-def linear_into(residual: Optional[torch.Tensor], x: torch.Tensor, weight: torch.Tensor) -> Optional[torch.Tensor]:
-    """``residual += x @ weight.T`` inside the product's kernel where that exists (few bfloat16
-    rows): then None is returned.  Otherwise the product is returned in float32 and the caller
-    hands it on to whoever adds it (the next norm's kernel)."""
-    m, k = x.shape
-    if (residual is not None and x.is_cuda and x.dtype == torch.bfloat16 and skinny.takes_resident(m, k, weight)
-            and residual.dtype == torch.float32 and residual.shape == (m, weight.shape[0]) and residual.stride(1) == 1
-            and x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0):
+def _aligned(x: torch.Tensor) -> bool:
+    return x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
+
+
+def linear_into(residual: Optional[torch.Tensor], x: torch.Tensor, weight: torch.Tensor,
+                swiglu: bool = False) -> Optional[torch.Tensor]:
+    """``residual += X @ weight.T`` inside the product's kernel where that exists (few bfloat16
+    rows): then None is returned.  Otherwise what is to be added is returned, in float32, and the
+    caller hands it on to whoever adds it (the next norm's kernel): the product ``[M, N]``, or
+    ``[slabs, M, N]`` whose slabs are added in order (17 to 64 rows whose inner size does not fit a
+    block: the chunked kernel).  With ``swiglu``, ``x`` is the grouped gate | up product ``[M, 2 K]``
+    and ``X = silu(gate) * up``."""
+    m = x.shape[0]
+    k = weight.shape[1]
+    fast = x.is_cuda and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and _aligned(x)
+    one_block = m <= 16 or (m <= skinny.ONE_BLOCK_ROWS and k <= skinny.resident_two_tile_k())
+    if fast and not one_block and skinny.takes_chunked(m, k, weight):
+        return skinny.chunked_product(weight, x, swiglu=swiglu)
+    if swiglu:
+        x = kernels.swiglu(x, grouped=True)
+    if (fast and one_block and residual is not None and skinny.takes_resident(m, k, weight)
+            and residual.dtype == torch.float32 and residual.shape == (m, weight.shape[0]) and residual.stride(1) == 1):
         skinny.resident_product(weight, x=x, epilogue=skinny.RESIDUAL, out=residual)
         return None
-    # More rows: the library's product.  Its bfloat16 output is the form it is tuned for (and the
-    # only one the tuner of `tune_library_products` covers); the sum into the residual stays float32.
-    return linear(x, weight, out_dtype=torch.float32 if x.shape[0] <= skinny.MAX_ROWS else None)
+    # More rows: the library's product, handed over in float32 like the fused kernel's sums, so that
+    # what joins the residual is rounded the same way however many tokens a step brings.
+    return linear(x, weight, out_dtype=torch.float32)
 
 
 def tune_library_products(enable: bool = True, max_ms: int = 3000) -> None:
@@ -106,11 +120,11 @@ def gate_up_swiglu(x: Union[torch.Tensor, NormedRows], weight: torch.Tensor, gro
     rows) or ``grouped`` (alternating groups of 8 gate rows and 8 up rows).  With few bfloat16 rows
     and grouped rows the activation is applied inside the product's kernel."""
     m, k = x.shape
-    if grouped and weight.dtype == torch.bfloat16 and weight.is_cuda and weight.shape[0] % 16 == 0:
+    if (grouped and weight.dtype == torch.bfloat16 and weight.is_cuda and weight.shape[0] % 16 == 0
+            and m <= skinny.ONE_BLOCK_ROWS):
         lazy = isinstance(x, NormedRows)
         if lazy and skinny.takes_resident(m, k, weight, norm=True):
             return skinny.resident_product(weight, h=x.h, norm_weight=x.weight, eps=x.eps, epilogue=skinny.SWIGLU)
-        if (not lazy and x.dtype == torch.bfloat16 and skinny.takes_resident(m, k, weight) and x.stride(1) == 1
-                and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0):
+        if not lazy and x.dtype == torch.bfloat16 and skinny.takes_resident(m, k, weight) and _aligned(x):
             return skinny.resident_product(weight, x=x, epilogue=skinny.SWIGLU)
     return kernels.swiglu(linear(x, weight), grouped=grouped)

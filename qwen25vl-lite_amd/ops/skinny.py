@@ -1,9 +1,9 @@
 """Dispatch of bfloat16 products with few rows to the hand-written kernels.
 
-Up to 32 rows: the resident kernel (``csrc/gemm_resident.hip``), which can also fold the RMSNorm
-before the product, the residual add after it, or the SwiGLU activation into itself; with 17 to 32
-rows it needs an inner size that fits one pass of a block.
-17 to 32 rows beyond that: the streaming kernel (``csrc/gemm_skinny.hip``) where it beats the library.
+Up to 64 rows: the resident kernel (``csrc/gemm_resident.hip``), which can also fold the RMSNorm
+before the product, the residual add after it, the SwiGLU activation, or the rotation and cache
+write into itself.  One block carries up to 32 rows; more rows (or 17 to 32 with a long inner
+size) are spread over teams of blocks that walk the same weight tiles on one XCD.
 """
 
 from __future__ import annotations
@@ -15,11 +15,13 @@ import torch
 
 from .kernels import _check, _fn, _ptr, _stream, dtype_code
 
-__all__ = ["resident_product", "takes_resident", "qkv_rope_product", "takes_qkv_rope", "try_streaming", "RESIDENT_ROWS", "resident_norm_k", "resident_two_tile_k", "folds_norm", "MAX_ROWS",
+__all__ = ["resident_product", "takes_resident", "qkv_rope_product", "takes_qkv_rope", "RESIDENT_ROWS", "resident_norm_k", "resident_two_tile_k", "folds_norm", "TEAM_LONG_K", "ONE_BLOCK_ROWS", "chunked_product", "takes_chunked", "CHUNKED_ROWS",
            "STORE", "RESIDUAL", "SWIGLU"]
 
-MAX_ROWS = 32            # the streaming kernel's limit in use
-RESIDENT_ROWS = 32       # up to here the resident kernel runs (one column tile of 16 rows, or two)
+RESIDENT_ROWS = 64       # up to here the resident kernel runs
+ONE_BLOCK_ROWS = 32      # up to here one block carries all rows: beyond, teams of blocks share the weight's
+                         # tiles, which pays for the fused q | k | v projection only
+TEAM_LONG_K = 1          # flag: 17 to 32 rows with a long inner size go to a team of two blocks
 _pass_k = None
 _two_tile_k = None
 STORE, RESIDUAL, SWIGLU = 0, 1, 2
@@ -56,30 +58,38 @@ def resident_two_tile_k() -> int:
     return _two_tile_k
 
 
-def folds_norm(m: int, k: int) -> bool:
-    """Whether the resident kernel forms the norm of ``m`` rows of width ``k`` by itself."""
-    return m <= RESIDENT_ROWS and k <= (resident_norm_k() if m <= 16 else resident_two_tile_k())
+def folds_norm(m: int, k: int, device=None) -> bool:
+    """Whether the resident kernel forms the norm of ``m`` rows of width ``k`` by itself (the
+    kernel's own rule: the rows must stay in their blocks for all of the weight's tiles)."""
+    if m > RESIDENT_ROWS or k % 8:
+        return False
+    fn = _fn("gemm_resident", "qvl_gemm_resident_folds_norm", [_c_int, _c_int, _c_int])
+    return bool(fn(int(m), int(k), _compute_units(device if device is not None else torch.cuda.current_device())))
 
 
 def takes_resident(m: int, k: int, weight: torch.Tensor, *, norm: bool = False) -> bool:
     """Whether the resident kernel takes a product of ``m`` rows with this weight, and is the
     better choice for it.  A K that fits one pass of the block always is (the rows stay in
-    registers for all of the block's tiles).  With a longer K the rows are read again for every
-    pass of every tile, which only pays while each compute unit has a single tile (at most
-    16 weight rows each): beyond that the library's product streams such a matrix faster
-    (measured at the 72B decoder's shapes, K of 8192 and 29568)."""
+    registers for all of the block's tiles), and so are 33 to 64 rows (teams of blocks with
+    resident rows).  Up to 32 rows with a longer K are read again for every pass of every tile,
+    which only pays while each compute unit has a single tile (at most 16 weight rows each):
+    beyond that the library's product streams such a matrix faster (measured at the 72B
+    decoder's shapes, K of 8192 and 29568)."""
     if m > RESIDENT_ROWS or k % 8 or weight.dtype != torch.bfloat16 or not _rows_aligned(weight, 8):
         return False
-    if k <= (resident_norm_k() if m <= 16 else resident_two_tile_k()):
+    if norm:
+        return folds_norm(m, k, weight.device)
+    if m > 32 or k <= (resident_norm_k() if m <= 16 else resident_two_tile_k()):
         return True
-    return not norm and weight.shape[0] <= 16 * _compute_units(weight.device)
+    return weight.shape[0] <= 16 * _compute_units(weight.device)
 
 
 def resident_product(weight: torch.Tensor, *, x: Optional[torch.Tensor] = None, h: Optional[torch.Tensor] = None,
                      norm_weight: Optional[torch.Tensor] = None, eps: float = 0.0,
                      bias: Optional[torch.Tensor] = None, epilogue: int = STORE,
-                     out: Optional[torch.Tensor] = None, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
-    """``X @ weight.T`` for at most 32 rows.  ``X`` is ``x`` (bfloat16), or ``rmsnorm(h) * norm_weight``
+                     out: Optional[torch.Tensor] = None, out_dtype: torch.dtype = torch.float32,
+                     flags: int = 0) -> torch.Tensor:
+    """``X @ weight.T`` for at most 64 rows (``h`` for at most 32).  ``X`` is ``x`` (bfloat16), or ``rmsnorm(h) * norm_weight``
     formed inside the kernel from the float32 rows ``h``.  ``epilogue``: ``STORE`` writes the product
     (plus ``bias``) to a new tensor of ``out_dtype``; ``RESIDUAL`` adds it to ``out`` (float32) in
     place; ``SWIGLU`` takes ``weight``'s rows as groups of 8 gate, 8 up rows and returns
@@ -108,10 +118,11 @@ def resident_product(weight: torch.Tensor, *, x: Optional[torch.Tensor] = None, 
         out, odt = torch.empty((m, n), dtype=out_dtype, device=src.device), out_dtype
     fn = _fn("gemm_resident", "qvl_gemm_resident",
              [_c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_float, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int,
-              _c_int, _c_int, _c_int, _c_int, _c_ptr])
+              _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
     _check(fn(_ptr(x), x.stride(0) if x is not None else 0, _ptr(h), h.stride(0) if h is not None else 0,
               _ptr(norm_weight), float(eps), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(out), out.stride(0),
-              m, n, k, dtype_code(odt), epilogue, _compute_units(src.device), _stream()), "linear (resident)")
+              m, n, k, dtype_code(odt), epilogue, _compute_units(src.device), int(flags), _stream()),
+           "linear (resident)")
     return out
 
 
@@ -128,7 +139,7 @@ def qkv_rope_product(weight: torch.Tensor, cs: torch.Tensor, *, x: Optional[torc
                      bias: Optional[torch.Tensor] = None, slots: Optional[torch.Tensor] = None,
                      k_cache: Optional[torch.Tensor] = None, v_cache: Optional[torch.Tensor] = None,
                      num_q_heads: int, num_kv_heads: int, head_dim: int, page_size: int) -> torch.Tensor:
-    """The stacked query | key | value projection of at most 32 tokens with the rotation and the
+    """The stacked query | key | value projection of at most 64 tokens with the rotation and the
     cache write inside the product's kernel: returns the rotated queries ``[M, nq hd]`` (bfloat16);
     rotated keys and values are in their page slots.  ``cs`` is :func:`kernels.rope_table` of the
     step's tokens.  With ``num_kv_heads == 0`` the weight holds query rows only."""
@@ -166,27 +177,33 @@ def qkv_rope_product(weight: torch.Tensor, cs: torch.Tensor, *, x: Optional[torc
     return q_out
 
 
-def prefers_streaming(m: int, n: int, k: int) -> bool:
-    """Where the streaming kernel (rows of x read again from L2 by every wave) beats the library's
-    product on MI355X, measured at the 7B decoder's shapes with 17 to 32 rows: the small square
-    matrix and the one with a long inner size."""
-    return 16 < m <= MAX_ROWS and (n * k <= 13_000_000 or k >= 4 * n)
+CHUNKED_ROWS = (17, 64)   # the rows the chunked kernel is built for
 
 
-def try_streaming(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
-                  out_dtype: Optional[torch.dtype]) -> Optional[torch.Tensor]:
-    """``x @ weight.T (+ bias)`` through the streaming kernel, or None if it is not the better choice
-    or does not take the shape."""
-    m, k = x.shape
-    n = weight.shape[0]
-    if not prefers_streaming(m, n, k) or k % 8 or not _rows_aligned(x, 8) or not _rows_aligned(weight, 8):
-        return None
-    if bias is not None and (bias.dtype != torch.float32 or not bias.is_contiguous() or bias.shape != (n,)):
-        return None
-    odt = out_dtype or x.dtype
-    out = torch.empty((m, n), dtype=odt, device=x.device)
-    fn = _fn("gemm_skinny", "qvl_gemm_skinny",
-             [_c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
-    _check(fn(_ptr(x), x.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(out), out.stride(0), m, n, k,
-              dtype_code(odt), _stream()), "linear (streaming)")
+def takes_chunked(m: int, k: int, weight: torch.Tensor) -> bool:
+    """Whether the chunked kernel (``csrc/gemm_chunked.hip``) takes a product of ``m`` rows with this
+    weight: 17 to 64 bfloat16 rows, whose partial sums over chunks of the inner size come back as
+    slabs."""
+    return (CHUNKED_ROWS[0] <= m <= CHUNKED_ROWS[1] and k % 8 == 0 and weight.dtype == torch.bfloat16
+            and _rows_aligned(weight, 8))
+
+
+def chunked_product(weight: torch.Tensor, x: torch.Tensor, *, swiglu: bool = False) -> torch.Tensor:
+    """Partial sums of ``X @ weight.T`` over chunks of the inner size: float32 ``[chunks, M, N]``,
+    whose sum over the first axis (taken in order by whoever reads them: the norm
+    that follows) is the product.  ``X`` is ``x`` (bfloat16 ``[M, K]``), or with ``swiglu`` ``x`` is
+    the grouped gate | up product ``[M, 2 K]`` and ``X = silu(gate) * up`` is formed on the way."""
+    m = x.shape[0]
+    n, k = weight.shape
+    if not takes_chunked(m, k, weight) or x.shape[1] != (2 * k if swiglu else k):
+        raise ValueError("the chunked kernel does not take this product")
+    if x.dtype != torch.bfloat16 or not _rows_aligned(x, 8):
+        raise ValueError("x must be bfloat16 with 16-byte aligned rows")
+    cus = _compute_units(x.device)
+    chunks = int(_fn("gemm_chunked", "qvl_gemm_chunked_chunks", [_c_int, _c_int, _c_int])(n, k, cus))
+    out = torch.empty((chunks, m, n), dtype=torch.float32, device=x.device)
+    fn = _fn("gemm_chunked", "qvl_gemm_chunked",
+             [_c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(x), x.stride(0), _ptr(weight), weight.stride(0), _ptr(out), m, n, k, int(swiglu), cus, _stream()),
+           "linear (chunked)")
     return out

@@ -36,7 +36,7 @@ class RMSNorm(Norm):
 
     def forward(self, stream: ResidualStream, rows: Optional[torch.Tensor] = None, lazy: bool = False):
         if (lazy and rows is None and stream.pending is None and self.dtype == torch.bfloat16
-                and self.size % 8 == 0 and skinny.folds_norm(stream.h.shape[0], self.size)):
+                and self.size % 8 == 0 and skinny.folds_norm(stream.h.shape[0], self.size, stream.h.device)):
             # a decode step: the product that follows computes the norm on the way
             return NormedRows(stream.h, self.weight, self.eps, self.dtype)
         out = kernels.add_rmsnorm(stream.h, stream.pending, self.weight, self.eps, self.dtype, rows=rows)

@@ -214,27 +214,31 @@ def test_decode_step_queued_ahead_changes_nothing(model_dirs, name, dtype):
         assert plain[3][0] == _plain_greedy(d, prompts[3], 8)
 
 
-@pytest.mark.parametrize("name, hip_graph", [("C_sharp", False), ("B_sharp", True)])
-def test_twenty_odd_requests_decode_together(model_dirs, name, hip_graph):
+@pytest.mark.parametrize("name, hip_graph, count", [("C_sharp", False, 21), ("B_sharp", True, 21), ("A_sharp", True, 52),
+                                                    ("C_sharp", False, 45)])
+def test_twenty_odd_requests_decode_together(model_dirs, name, hip_graph, count):
     """Between 17 and 32 decoded tokens a step the bfloat16 products run with two column tiles of
-    rows (norm, rotation with cache write, activation and residual folded in as with fewer): 21
-    requests of different lengths, some ending early so that the batch shrinks through 24, 16 and
+    rows (norm, rotation with cache write, activation and residual folded in as with fewer), and
+    between 33 and 64 with teams of blocks for the fused q | k | v projection and the kernel that
+    cuts the inner size for the output and down projections: 21, 45 or 52
+    requests of different lengths, some ending early so that the batch shrinks through 48, 32, 24, 16 and
     12 rows.  float32 gives the plain implementation's tokens.  bfloat16 gives them up to the first
     place where the plain logits' two best lie closer than the bound on bfloat16 logits (2e-2, as
-    in the replay tests): there either token is right, and what follows it is another sequence."""
+    in the replay tests): there the token the engine picked lies within that bound of the best, and
+    what follows it is another sequence."""
     from qwen25vl_lite_amd import LLM, SamplingParams
 
     d = model_dirs[name]
-    vocab = {"B": 509, "C": 300}[name[0]]
-    prompts = [random_tokens(3 + (5 * i) % 23, vocab, 300 + i) for i in range(21)]
-    params = [SamplingParams(temperature=0.0, max_tokens=4 + (7 * i) % 19, ignore_eos=True) for i in range(21)]
-    common = dict(num_blocks=128, block_size=16, max_num_seqs=32, max_num_batched_tokens=512,
+    vocab = {"A": 256, "B": 509, "C": 300}[name[0]]
+    prompts = [random_tokens(3 + (5 * i) % 23, vocab, 300 + i) for i in range(count)]
+    params = [SamplingParams(temperature=0.0, max_tokens=4 + (7 * i) % 19, ignore_eos=True) for i in range(count)]
+    common = dict(num_blocks=256, block_size=16, max_num_seqs=64, max_num_batched_tokens=1024,
                   enable_prefix_cache=False, hip_graph=hip_graph)
     exact = LLM(d, dtype="float32", **common).generate(prompts, params)
     llm = LLM(d, dtype="bfloat16", **common)
     outs = llm.generate(prompts, params)
     if hip_graph:
-        assert 24 in {k[0] for k in llm.runner.graphs.graphs}
+        assert (24 if count < 32 else 48) in {k[0] for k in llm.runner.graphs.graphs}
     whole = 0
     for prompt, out, ex, p in zip(prompts, outs, exact, params):
         want = _plain_greedy(d, prompt, p.max_tokens)
@@ -244,9 +248,9 @@ def test_twenty_odd_requests_decode_together(model_dirs, name, hip_graph):
             whole += 1
             continue
         j = next(k for k in range(len(want)) if got[k] != want[k])
-        best = torch.topk(plain_model_logits(d, list(prompt) + want[:j])[-1], 2)
-        assert got[j] == int(best.indices[1]) and float(best.values[0] - best.values[1]) < 2e-2, (j, best)
-    assert whole >= 14          # ties are the exception
+        row = plain_model_logits(d, list(prompt) + want[:j])[-1]
+        assert float(row.max() - row[got[j]]) < 2e-2, (j, torch.topk(row, 3), got[j])
+    assert whole >= count * 2 // 3          # ties are the exception
     assert llm.runner.cache.pages_in_use() == [0] * len(llm.runner.cache.groups)
 
 

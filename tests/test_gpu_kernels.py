@@ -281,12 +281,13 @@ def test_gemm_f32_is_exact_and_row_independent(m, n, k):
 @pytest.mark.parametrize("m, n, k", [(1, 509, 144), (8, 300, 200), (16, 17, 8), (9, 100, 8200), (17, 1000, 4104),
                                      (31, 130, 352), (64, 509, 3584), (5, 40, 100), (300, 64, 1000),
                                      (17, 4700, 3584), (32, 300, 3840), (24, 509, 3848), (20, 33, 8),
-                                     (30, 4104, 4000), (16, 4104, 4104)])
+                                     (30, 4104, 4000), (16, 4104, 4104), (33, 300, 200), (64, 4700, 3584),
+                                     (48, 509, 3848), (41, 130, 8200), (64, 3584, 18944), (65, 300, 200)])
 def test_linear_bfloat16(m, n, k):
-    """Up to 32 rows go through the resident matrix-core kernel (inner sizes in steps of 8): always
-    if the inner size fits one pass of a block (4096, or 3840 with 17 to 32 rows), and with a longer
-    one while each compute unit has one tile at most; the rest through the streaming kernel
-    (17 to 32 rows, where it wins) or the library; all accumulate in float32."""
+    """Up to 64 rows go through the resident matrix-core kernel (inner sizes in steps of 8): up to 32
+    rows always if the inner size fits one pass of a block (4096, or 3840 with 17 to 32 rows), and
+    with a longer one while each compute unit has one tile at most; 33 to 64 rows always (their
+    rows are streamed); the rest through the library; all accumulate in float32."""
     from qwen25vl_lite_amd.ops import skinny
     from qwen25vl_lite_amd.ops.linear import linear
     torch.manual_seed(k)
@@ -295,7 +296,7 @@ def test_linear_bfloat16(m, n, k):
     want = x.float() @ w.float().T
     units = torch.cuda.get_device_properties(0).multi_processor_count
     assert skinny.takes_resident(m, k, w.cuda()) == (
-        k % 8 == 0 and m <= 32 and (k <= (4096 if m <= 16 else 3840) or n <= 16 * units))
+        k % 8 == 0 and m <= 64 and (m > 32 or k <= (4096 if m <= 16 else 3840) or n <= 16 * units))
     out32 = linear(x.cuda(), w.cuda(), out_dtype=torch.float32)
     assert out32.dtype == torch.float32 and torch.allclose(out32.cpu(), want, atol=2e-3, rtol=2e-3)
     out16 = linear(x.cuda(), w.cuda())
@@ -309,7 +310,8 @@ def test_linear_bfloat16(m, n, k):
 
 
 @pytest.mark.parametrize("m, n, k", [(1, 48, 64), (7, 1000, 3584), (16, 130, 4096), (3, 64, 144),
-                                     (17, 1000, 3584), (32, 130, 3840), (29, 64, 144), (24, 48, 4096)])
+                                     (17, 1000, 3584), (32, 130, 3840), (29, 64, 144), (24, 48, 4096),
+                                     (33, 1000, 3584), (64, 64, 144)])
 def test_product_with_the_norm_folded_in(m, n, k):
     """rmsnorm(h) * w formed inside the product equals the norm kernel followed by the product."""
     from qwen25vl_lite_amd.ops import kernels
@@ -323,6 +325,13 @@ def test_product_with_the_norm_folded_in(m, n, k):
     want = plain_rmsnorm(h.cpu(), g.cpu(), 1e-5).bfloat16().float() @ w.float().cpu().T
     assert torch.allclose(fused.cpu(), want, atol=3e-3, rtol=3e-3)
     assert (fused - apart).abs().max() < 0.02 * want.abs().max()   # the same up to a bfloat16 rounding of x here and there
+    if m > 32:   # teams of blocks: `linear` leaves these to the library, the kernel itself takes them
+        from qwen25vl_lite_amd.ops import skinny
+        assert skinny.folds_norm(m, k)
+        team = skinny.resident_product(w, h=h, norm_weight=g, eps=1e-5, out_dtype=torch.float32)
+        assert torch.allclose(team.cpu(), want, atol=3e-3, rtol=3e-3)
+        both = skinny.resident_product(w, x=kernels.add_rmsnorm(h, None, g, 1e-5, torch.bfloat16), out_dtype=torch.float32)
+        assert torch.allclose(both.cpu(), want, atol=3e-3, rtol=3e-3)
     # a longer row than one pass of the block holds is computed by the norm's own kernel first
     h2, g2 = torch.randn(2, 4104).cuda(), torch.ones(4104).cuda()
     w2 = (torch.randn(24, 4104) / 64).bfloat16().cuda()
@@ -332,7 +341,8 @@ def test_product_with_the_norm_folded_in(m, n, k):
 
 
 @pytest.mark.parametrize("m, n, k", [(1, 144, 352), (8, 3584, 18944), (16, 100, 4104), (24, 144, 352), (40, 144, 352),
-                                     (32, 3584, 3584), (17, 100, 3840), (24, 144, 4104), (32, 3584, 18944)])
+                                     (32, 3584, 3584), (17, 100, 3840), (24, 144, 4104), (32, 3584, 18944),
+                                     (64, 3584, 18944), (33, 3584, 3584), (57, 100, 4104), (70, 144, 352)])
 def test_product_added_into_the_residual(m, n, k):
     from qwen25vl_lite_amd.ops.linear import linear_into
     torch.manual_seed(k)
@@ -341,18 +351,21 @@ def test_product_added_into_the_residual(m, n, k):
     h = torch.randn(m, n).cuda()
     want = h.cpu() + x.float().cpu() @ w.float().cpu().T
     left = linear_into(h, x, w)
-    if m <= 32:
+    if m <= 16 or (m <= 32 and k <= 3840):      # one block carries the rows: added in place
         assert left is None and torch.allclose(h.cpu(), want, atol=3e-3, rtol=3e-3)
-    else:   # too many rows for the fused kernel: the library's product comes back in bfloat16 for
-        # the next norm to add
-        assert left is not None and left.dtype == torch.bfloat16
-        assert torch.allclose(h.cpu() + left.float().cpu(), want, atol=2e-2, rtol=2e-2)
+    elif m <= 64:   # the chunked kernel: slabs of partial sums for the next norm to add
+        assert left.dtype == torch.float32 and left.dim() == 3 and tuple(left.shape[1:]) == (m, n)
+        assert torch.allclose(h.cpu() + left.sum(0).cpu(), want, atol=3e-3, rtol=3e-3)
+    else:   # the library's product comes back, in float32 too
+        assert left is not None and left.dtype == torch.float32 and left.dim() == 2
+        assert torch.allclose(h.cpu() + left.cpu(), want, atol=3e-3, rtol=3e-3)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("m, inter, k", [(1, 352, 144), (8, 18944, 3584), (16, 40, 4104), (50, 352, 144),
                                          (4, 2072, 64), (3, 5136, 72), (2, 8 * 320, 40),
-                                         (32, 18944, 3584), (17, 2072, 64), (25, 5136, 72)])
+                                         (32, 18944, 3584), (17, 2072, 64), (25, 5136, 72), (64, 18944, 3584),
+                                         (33, 2072, 64), (47, 5136, 72), (70, 352, 144)])
 def test_gate_up_product_with_the_activation_folded_in(dtype, m, inter, k):
     """Grouped gate | up rows: few bfloat16 rows get silu(gate) * up from the product's own kernel,
     everything else from the product followed by the activation kernel on the grouped columns."""
@@ -371,6 +384,45 @@ def test_gate_up_product_with_the_activation_folded_in(dtype, m, inter, k):
     assert torch.allclose(plain.float().cpu(), want, **tol)
 
 
+@pytest.mark.parametrize("m, n, k, swiglu", [(64, 3584, 18944, True), (17, 509, 352, False), (33, 130, 200, False),
+                                             (48, 1000, 3584, False), (40, 144, 352, True), (64, 37, 8, False),
+                                             (25, 4700, 1248, True), (57, 300, 1256, False)])
+def test_chunked_product_and_the_norm_that_adds_its_slabs(m, n, k, swiglu):
+    """17 to 64 rows against a weight cut along its inner size: the slabs of partial sums add up to
+    the product (inner sizes that are no multiple of 32, row counts that fill no tile), with the
+    activation applied while the rows are fetched if asked, twice the same bits; and the norm
+    kernel that takes the slabs as its addend gives what it gives for their sum."""
+    from qwen25vl_lite_amd.ops import kernels, skinny
+    torch.manual_seed(n + k)
+    w = (torch.randn(n, k) / math.sqrt(k)).bfloat16()
+    if swiglu:
+        gate, up = torch.randn(m, k).bfloat16(), torch.randn(m, k).bfloat16()
+        x_in = torch.stack([gate.view(m, -1, 8), up.view(m, -1, 8)], dim=2).reshape(m, 2 * k).contiguous()
+        x = (torch.nn.functional.silu(gate.float()) * up.float()).bfloat16()
+    else:
+        x = x_in = torch.randn(m, k).bfloat16()
+    want = x.float() @ w.float().T
+    assert skinny.takes_chunked(m, k, w.cuda()) and not skinny.takes_chunked(16, k, w.cuda())
+    slabs = skinny.chunked_product(w.cuda(), x_in.cuda(), swiglu=swiglu)
+    assert slabs.dtype == torch.float32 and slabs.dim() == 3 and tuple(slabs.shape[1:]) == (m, n)
+    assert torch.allclose(slabs.sum(0).cpu(), want, atol=3e-3, rtol=3e-3), (slabs.sum(0).cpu() - want).abs().max()
+    assert torch.equal(slabs, skinny.chunked_product(w.cuda(), x_in.cuda(), swiglu=swiglu))
+    if n % 4 == 0:
+        h = torch.randn(m, n).cuda()
+        g = (1 + 0.1 * torch.randn(n)).cuda()
+        h1, h2 = h.clone(), h.clone()
+        a = kernels.add_rmsnorm(h1, slabs, g, 1e-6, torch.bfloat16)
+        total = slabs[0].clone()
+        for c in range(1, slabs.shape[0]):
+            total += slabs[c]
+        b = kernels.add_rmsnorm(h2, total, g, 1e-6, torch.bfloat16)
+        assert torch.equal(h1, h2) and torch.equal(a, b), "the slabs are added in their order"
+        rows = torch.tensor([m - 1, 0], dtype=torch.int32).cuda()
+        h3 = h.clone()
+        c3 = kernels.add_rmsnorm(h3, slabs, g, 1e-6, torch.float32, rows=rows)
+        assert torch.equal(h3, h) and torch.allclose(c3, kernels.add_rmsnorm(h.clone(), total, g, 1e-6, torch.float32)[[m - 1, 0]])
+
+
 def test_no_cpu_path():
     from qwen25vl_lite_amd.ops import kernels
     from qwen25vl_lite_amd.ops.linear import linear
@@ -386,7 +438,8 @@ def test_no_cpu_path():
 @pytest.mark.parametrize("m, nq, nkv, hd, k, bias, lazy", [(1, 4, 2, 16, 64, True, False), (8, 28, 4, 128, 3584, True, True),
                                                          (16, 6, 3, 48, 136, False, True), (5, 3, 0, 80, 104, True, False),
                                                          (32, 28, 4, 128, 3584, True, True), (17, 6, 3, 48, 136, False, True),
-                                                         (27, 4, 2, 16, 64, True, False)])
+                                                         (27, 4, 2, 16, 64, True, False), (64, 28, 4, 128, 3584, True, False),
+                                                         (33, 6, 3, 48, 136, False, False), (50, 4, 2, 16, 64, True, False)])
 def test_projection_with_rotation_and_cache_write_folded_in(m, nq, nkv, hd, k, bias, lazy, ps):
     """The stacked q | k | v projection of a few rows that rotates and stores inside the product's
     kernel equals the product followed by the rotation kernel: queries, and every slot of the
