@@ -96,8 +96,7 @@ template <> __device__ __forceinline__ void st4<bf16_t>(bf16_t* p, float4 v) {
 template <typename TD, typename TO>
 __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict__ h, const TD* __restrict__ delta,
                                                               const float* __restrict__ w, TO* __restrict__ out,
-                                                              const int* __restrict__ rows, int H, float eps,
-                                                              int nslabs, long long slab_stride) {
+                                                              const int* __restrict__ rows, int H, float eps) {
   __shared__ float red[17];
   const int m = blockIdx.x;
   const int row = rows ? rows[m] : m;
@@ -112,11 +111,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
     if (i < nvec) {
       float4 x = ld4<float>(hr + 4 * i);
       if (dr) {
-        float4 d = ld4<TD>(dr + 4 * i);
-        for (int c = 1; c < nslabs; ++c) {
-          const float4 e = ld4<TD>(dr + (size_t)c * slab_stride + 4 * i);
-          d.x += e.x; d.y += e.y; d.z += e.z; d.w += e.w;
-        }
+        const float4 d = ld4<TD>(dr + 4 * i);
         x.x += d.x; x.y += d.y; x.z += d.z; x.w += d.w;
         if (!rows) st4<float>(hr + 4 * i, x);
       }
@@ -136,6 +131,58 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
   }
 }
 
+// The addend as slabs of partial sums (float32 [slab][row][H], H a multiple of 4 and at most
+// SLAB_VEC_MAX * 4096): a block of 1024 threads per row, a thread per 4 neighbouring values, the
+// slabs' loads asked for eight at a time (they do not depend on each other, only the sum has an
+// order: slab 0, 1, 2, ...).
+#define SLAB_VEC_MAX 2
+template <typename TO>
+__global__ __launch_bounds__(1024) void add_rmsnorm_slabs_kernel(float* __restrict__ h, const float* __restrict__ delta,
+                                                                 const float* __restrict__ w, TO* __restrict__ out,
+                                                                 const int* __restrict__ rows, int H, float eps,
+                                                                 int nslabs, long long slab_stride) {
+  __shared__ float red[17];
+  const int m = blockIdx.x;
+  const int row = rows ? rows[m] : m;
+  float* hr = h + (size_t)row * H;
+  const float* dr = delta + (size_t)row * H;
+  const int nvec = H >> 2;
+  float4 v[SLAB_VEC_MAX];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < SLAB_VEC_MAX; ++j) {
+    const int i = threadIdx.x + 1024 * j;
+    if (i < nvec) {
+      float4 d = {0.f, 0.f, 0.f, 0.f};
+      for (int c0 = 0; c0 < nslabs; c0 += 8) {
+        float4 e[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+          e[c] = c0 + c < nslabs ? ld4<float>(dr + (size_t)(c0 + c) * slab_stride + 4 * i) : float4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+          if (c0 + c < nslabs) { d.x += e[c].x; d.y += e[c].y; d.z += e[c].z; d.w += e[c].w; }
+        }
+      }
+      float4 x = ld4<float>(hr + 4 * i);
+      x.x += d.x; x.y += d.y; x.z += d.z; x.w += d.w;
+      if (!rows) st4<float>(hr + 4 * i, x);
+      v[j] = x;
+      ss += x.x * x.x + x.y * x.y + x.z * x.z + x.w * x.w;
+    }
+  }
+  const float rs = 1.0f / sqrtf(block_sum(ss, red) / (float)H + eps);
+  TO* o = out + (size_t)m * H;
+#pragma unroll
+  for (int j = 0; j < SLAB_VEC_MAX; ++j) {
+    const int i = threadIdx.x + 1024 * j;
+    if (i < nvec) {
+      const float4 g = ld4<float>(w + 4 * i);
+      st4<TO>(o + 4 * i, float4{(v[j].x * rs) * g.x, (v[j].y * rs) * g.y, (v[j].z * rs) * g.z, (v[j].w * rs) * g.w});
+    }
+  }
+}
+
 // delta: null, or nslabs slabs of [rows of h][H], slab_stride elements apart (nslabs 1: one addend).
 extern "C" int qvl_add_rmsnorm(void* h, const void* delta, const void* w, void* out, const void* rows, int M, int H,
                                float eps, int delta_dtype, int out_dtype, int nslabs, long long slab_stride,
@@ -143,13 +190,23 @@ extern "C" int qvl_add_rmsnorm(void* h, const void* delta, const void* w, void* 
   if (M <= 0) return QVL_OK;
   if (H <= 0 || nslabs < 1 || (nslabs > 1 && (slab_stride < H || slab_stride % 4))) return QVL_ERR_SHAPE;
   const int threads = H >= 2048 ? 512 : 256;
-  const bool vec = H % 4 == 0 && H <= NORM_VEC_MAX * 4 * 256;
+  const bool vec = H % 4 == 0 && H <= NORM_VEC_MAX * 4 * 256 && nslabs == 1;
+  if (nslabs > 1 && delta && delta_dtype == 0 && H % 4 == 0 && H <= SLAB_VEC_MAX * 4096) {
+    if (out_dtype == 0)
+      hipLaunchKernelGGL((add_rmsnorm_slabs_kernel<float>), dim3(M), dim3(1024), 0, stream, (float*)h, (const float*)delta,
+                         (const float*)w, (float*)out, (const int*)rows, H, eps, nslabs, slab_stride);
+    else if (out_dtype == 1)
+      hipLaunchKernelGGL((add_rmsnorm_slabs_kernel<bf16_t>), dim3(M), dim3(1024), 0, stream, (float*)h, (const float*)delta,
+                         (const float*)w, (bf16_t*)out, (const int*)rows, H, eps, nslabs, slab_stride);
+    else
+      return QVL_ERR_DTYPE;
+    return qvl_launch_status();
+  }
 #define QVL_NORM_CASE(DD, OD, TD, TO)                                                                              \
   if (delta_dtype == DD && out_dtype == OD) {                                                                      \
     if (vec)                                                                                                       \
       hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TO>), dim3(M), dim3(256), 0, stream, (float*)h,               \
-                         (const TD*)delta, (const float*)w, (TO*)out, (const int*)rows, H, eps, nslabs,            \
-                         slab_stride);                                                                             \
+                         (const TD*)delta, (const float*)w, (TO*)out, (const int*)rows, H, eps);                   \
     else                                                                                                           \
       hipLaunchKernelGGL((add_rmsnorm_kernel<TD, TO>), dim3(M), dim3(threads), 0, stream, (float*)h,               \
                          (const TD*)delta, (const float*)w, (TO*)out, (const int*)rows, H, eps, nslabs,            \

@@ -73,29 +73,22 @@ def _aligned(x: torch.Tensor) -> bool:
     return x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
 
 
-def linear_into(residual: Optional[torch.Tensor], x: torch.Tensor, weight: torch.Tensor,
-                swiglu: bool = False) -> Optional[torch.Tensor]:
-    """``residual += X @ weight.T`` inside the product's kernel where that exists (few bfloat16
-    rows): then None is returned.  Otherwise what is to be added is returned, in float32, and the
-    caller hands it on to whoever adds it (the next norm's kernel): the product ``[M, N]``, or
-    ``[slabs, M, N]`` whose slabs are added in order (17 to 64 rows whose inner size does not fit a
-    block: the chunked kernel).  With ``swiglu``, ``x`` is the grouped gate | up product ``[M, 2 K]``
-    and ``X = silu(gate) * up``."""
-    m = x.shape[0]
-    k = weight.shape[1]
+def linear_into(residual: Optional[torch.Tensor], x: torch.Tensor, weight: torch.Tensor) -> Optional[torch.Tensor]:
+    """``residual += x @ weight.T`` inside the product's kernel where that exists (few bfloat16
+    rows): then None is returned.  Otherwise what is to be added is returned and the caller hands
+    it on to whoever adds it (the next norm's kernel): the product ``[M, N]``, or float32
+    ``[slabs, M, N]`` whose slabs are added in order (the chunked kernel)."""
+    m, k = x.shape
     fast = x.is_cuda and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and _aligned(x)
-    one_block = m <= 16 or (m <= skinny.ONE_BLOCK_ROWS and k <= skinny.resident_two_tile_k())
-    if fast and not one_block and skinny.takes_chunked(m, k, weight):
-        return skinny.chunked_product(weight, x, swiglu=swiglu)
-    if swiglu:
-        x = kernels.swiglu(x, grouped=True)
-    if (fast and one_block and residual is not None and skinny.takes_resident(m, k, weight)
+    if fast and skinny.prefers_chunked(m, k, weight):
+        return skinny.chunked_product(weight, x)
+    if (fast and m <= skinny.ONE_BLOCK_ROWS and residual is not None and skinny.takes_resident(m, k, weight)
             and residual.dtype == torch.float32 and residual.shape == (m, weight.shape[0]) and residual.stride(1) == 1):
         skinny.resident_product(weight, x=x, epilogue=skinny.RESIDUAL, out=residual)
         return None
-    # More rows: the library's product, handed over in float32 like the fused kernel's sums, so that
-    # what joins the residual is rounded the same way however many tokens a step brings.
-    return linear(x, weight, out_dtype=torch.float32)
+    # More rows: the library's product.  Its bfloat16 output is the form it is tuned for (float32
+    # output costs a tenth of a 2,048-token prefill); the sum into the residual stays float32.
+    return linear(x, weight, out_dtype=torch.float32 if m <= skinny.ONE_BLOCK_ROWS else None)
 
 
 def tune_library_products(enable: bool = True, max_ms: int = 3000) -> None:

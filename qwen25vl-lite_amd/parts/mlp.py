@@ -6,8 +6,7 @@ from typing import Dict, Optional
 
 import torch
 
-from ..ops import skinny
-from ..ops.linear import gate_up_swiglu, linear, linear_into
+from ..ops.linear import gate_up_swiglu, linear_into
 from .base import FeedForward, ParamSpec, StepContext, register_part
 
 __all__ = ["SwiGLU"]
@@ -58,15 +57,8 @@ class SwiGLU(FeedForward):
         return {"gate_proj.weight": gate, "up_proj.weight": up, "down_proj.weight": self.w_down}
 
     def forward(self, x, step: StepContext):
-        residual = step.residual if step is not None else None
-        m = x.shape[0]
-        if (self.grouped and self.dtype == torch.bfloat16 and m > skinny.ONE_BLOCK_ROWS
-                and skinny.takes_chunked(m, self.inter, self.w_down)):
-            # 33 to 64 rows: the library's gate | up product, whose activation the down projection's
-            # kernel applies while it fetches its rows
-            return linear_into(residual, linear(x, self.w_gate_up), self.w_down, swiglu=True)
         act = gate_up_swiglu(x, self.w_gate_up, self.grouped)
-        return linear_into(residual, act, self.w_down)
+        return linear_into(step.residual if step is not None else None, act, self.w_down)
 
 
 register_part("ffn", "swiglu", SwiGLU)

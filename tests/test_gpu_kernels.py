@@ -353,12 +353,12 @@ def test_product_added_into_the_residual(m, n, k):
     left = linear_into(h, x, w)
     if m <= 16 or (m <= 32 and k <= 3840):      # one block carries the rows: added in place
         assert left is None and torch.allclose(h.cpu(), want, atol=3e-3, rtol=3e-3)
-    elif m <= 64:   # the chunked kernel: slabs of partial sums for the next norm to add
+    elif m <= 32 or (m <= 64 and n * k <= 1 << 24):   # the chunked kernel: slabs of partial sums for the next norm to add
         assert left.dtype == torch.float32 and left.dim() == 3 and tuple(left.shape[1:]) == (m, n)
         assert torch.allclose(h.cpu() + left.sum(0).cpu(), want, atol=3e-3, rtol=3e-3)
-    else:   # the library's product comes back, in float32 too
-        assert left is not None and left.dtype == torch.float32 and left.dim() == 2
-        assert torch.allclose(h.cpu() + left.cpu(), want, atol=3e-3, rtol=3e-3)
+    else:   # the library's product comes back in bfloat16 for the next norm to add
+        assert left is not None and left.dtype == torch.bfloat16 and left.dim() == 2
+        assert torch.allclose(h.cpu() + left.float().cpu(), want, atol=2e-2, rtol=2e-2)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -384,29 +384,23 @@ def test_gate_up_product_with_the_activation_folded_in(dtype, m, inter, k):
     assert torch.allclose(plain.float().cpu(), want, **tol)
 
 
-@pytest.mark.parametrize("m, n, k, swiglu", [(64, 3584, 18944, True), (17, 509, 352, False), (33, 130, 200, False),
-                                             (48, 1000, 3584, False), (40, 144, 352, True), (64, 37, 8, False),
-                                             (25, 4700, 1248, True), (57, 300, 1256, False)])
-def test_chunked_product_and_the_norm_that_adds_its_slabs(m, n, k, swiglu):
+@pytest.mark.parametrize("m, n, k", [(64, 3584, 18944), (17, 509, 352), (33, 130, 200), (48, 1000, 3584), (40, 144, 352),
+                                     (64, 37, 8), (25, 4700, 1248), (57, 300, 1256)])
+def test_chunked_product_and_the_norm_that_adds_its_slabs(m, n, k):
     """17 to 64 rows against a weight cut along its inner size: the slabs of partial sums add up to
-    the product (inner sizes that are no multiple of 32, row counts that fill no tile), with the
-    activation applied while the rows are fetched if asked, twice the same bits; and the norm
-    kernel that takes the slabs as its addend gives what it gives for their sum."""
+    the product (inner sizes that are no multiple of 32, row counts that fill no tile), twice the
+    same bits; and the norm kernel that takes the slabs as its addend gives what it gives for
+    their sum."""
     from qwen25vl_lite_amd.ops import kernels, skinny
     torch.manual_seed(n + k)
     w = (torch.randn(n, k) / math.sqrt(k)).bfloat16()
-    if swiglu:
-        gate, up = torch.randn(m, k).bfloat16(), torch.randn(m, k).bfloat16()
-        x_in = torch.stack([gate.view(m, -1, 8), up.view(m, -1, 8)], dim=2).reshape(m, 2 * k).contiguous()
-        x = (torch.nn.functional.silu(gate.float()) * up.float()).bfloat16()
-    else:
-        x = x_in = torch.randn(m, k).bfloat16()
+    x = torch.randn(m, k).bfloat16()
     want = x.float() @ w.float().T
     assert skinny.takes_chunked(m, k, w.cuda()) and not skinny.takes_chunked(16, k, w.cuda())
-    slabs = skinny.chunked_product(w.cuda(), x_in.cuda(), swiglu=swiglu)
+    slabs = skinny.chunked_product(w.cuda(), x.cuda())
     assert slabs.dtype == torch.float32 and slabs.dim() == 3 and tuple(slabs.shape[1:]) == (m, n)
     assert torch.allclose(slabs.sum(0).cpu(), want, atol=3e-3, rtol=3e-3), (slabs.sum(0).cpu() - want).abs().max()
-    assert torch.equal(slabs, skinny.chunked_product(w.cuda(), x_in.cuda(), swiglu=swiglu))
+    assert torch.equal(slabs, skinny.chunked_product(w.cuda(), x.cuda()))
     if n % 4 == 0:
         h = torch.randn(m, n).cuda()
         g = (1 + 0.1 * torch.randn(n)).cuda()
@@ -416,7 +410,9 @@ def test_chunked_product_and_the_norm_that_adds_its_slabs(m, n, k, swiglu):
         for c in range(1, slabs.shape[0]):
             total += slabs[c]
         b = kernels.add_rmsnorm(h2, total, g, 1e-6, torch.bfloat16)
-        assert torch.equal(h1, h2) and torch.equal(a, b), "the slabs are added in their order"
+        assert torch.equal(h1, h2), "the slabs are added in their order"
+        # (the two kernels add the squares up in different orders: the scale may differ in its last bit)
+        assert torch.allclose(a.float(), b.float(), atol=1e-2, rtol=1e-2)
         rows = torch.tensor([m - 1, 0], dtype=torch.int32).cuda()
         h3 = h.clone()
         c3 = kernels.add_rmsnorm(h3, slabs, g, 1e-6, torch.float32, rows=rows)
