@@ -71,6 +71,62 @@ def prefill_flops(t, tokens):
     return linear + attention + head
 
 
+def measure_peaks(torch):
+    """Plain read and copy rates, the matrix instruction's rate on registers and the cost of an empty
+    launch, each the best of several repeats (kernels in qwen25vl-lite_amd/csrc/peaks.hip)."""
+    import ctypes
+
+    from qwen25vl_lite_amd.ops.kernels import _check, _fn, _stream
+
+    c_int, c_ptr, c_ll = ctypes.c_int, ctypes.c_void_p, ctypes.c_longlong
+    read = _fn("peaks", "qvl_peak_read", [c_ptr, c_ll, c_ptr, c_int, c_ptr])
+    copy = _fn("peaks", "qvl_peak_copy", [c_ptr, c_ptr, c_ll, c_int, c_ptr])
+    mfma = _fn("peaks", "qvl_peak_mfma", [c_ptr, c_int, c_int, c_ptr])
+    empty = _fn("peaks", "qvl_peak_empty", [c_int, c_ptr])
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+
+    def best_ms(fn, reps=7):
+        fn()
+        torch.cuda.synchronize()
+        best = 1e9
+        for _ in range(reps):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            fn()
+            b.record()
+            torch.cuda.synchronize()
+            best = min(best, a.elapsed_time(b))
+        return best
+
+    out = {"device": torch.cuda.get_device_name(0), "compute_units": cus}
+    flag = torch.zeros(64, dtype=torch.int32, device="cuda")
+    for mib in (256, 1024, 4096):      # below and above the 256 MiB memory-side cache
+        nbytes = mib << 20
+        src = torch.empty(nbytes, dtype=torch.uint8, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        ms = best_ms(lambda: _check(read(src.data_ptr(), nbytes // 16, flag.data_ptr(), cus * 8, _stream()), "read"))
+        out[f"read_{mib}MiB_TBps"] = round(nbytes / ms / 1e9, 3)
+        ms = best_ms(lambda: _check(copy(src.data_ptr(), dst.data_ptr(), nbytes // 16, cus * 8, _stream()), "copy"))
+        out[f"copy_{mib}MiB_read_plus_write_TBps"] = round(2 * nbytes / ms / 1e9, 3)
+        ms = best_ms(lambda: dst.copy_(src))
+        out[f"device_to_device_copy_{mib}MiB_read_plus_write_TBps"] = round(2 * nbytes / ms / 1e9, 3)
+        del src, dst
+    iters, blocks = 4096, cus * 8
+    ms = best_ms(lambda: _check(mfma(flag.data_ptr(), iters, blocks, _stream()), "mfma"))
+    flops = blocks * 4 * iters * 8 * 2.0 * 16 * 16 * 32
+    out["mfma_16x16x32_bf16_PFLOPs"] = round(flops / ms / 1e12, 3)
+    # an empty kernel many times in a row, from the host and from a graph
+    n = 200
+    ms = best_ms(lambda: _check(empty(n, _stream()), "empty"))
+    out["empty_launch_from_host_us"] = round(ms * 1e3 / n, 2)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        _check(empty(n, _stream()), "empty")
+    ms = best_ms(graph.replay)
+    out["empty_launch_in_graph_us"] = round(ms * 1e3 / n, 2)
+    return out
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -86,6 +142,9 @@ def main(argv=None) -> int:
     ap.add_argument("--serving", action="store_true",
                     help="instead: continuous batching of 64 requests (prompts "
                          "of 64 to 2048 tokens, 32 to 512 generated, a quarter sharing a 1024-token prefix)")
+    ap.add_argument("--peaks", action="store_true",
+                    help="instead: what the device does at best (plain reads and copies, matrix instructions on "
+                         "registers, an empty launch), for the fractions above to be read against")
     ap.add_argument("--no-graph", action="store_true", help="do not replay decode steps from a HIP graph")
     ap.add_argument("--no-lookahead", action="store_true",
                     help="do not queue the next decode step before the running one's tokens are known")
@@ -96,6 +155,10 @@ def main(argv=None) -> int:
         return 2
 
     import torch
+
+    if args.peaks:
+        print(json.dumps(measure_peaks(torch)))
+        return 0
 
     from qwen25vl_lite_amd import EngineConfig, LLMEngine, ModelRunner, Qwen25VLConfig, SamplingParams, build_model
     from qwen25vl_lite_amd.config import dtype_from_name

@@ -17,6 +17,7 @@ LIBRARIES = [
     ("sample", {}),
     ("gemm_resident", {}),
     ("gemm_chunked", {}),
+    ("peaks", {}),
     # the matrix-core attention is compiled per head size; these are the sizes the tests and the
     # benchmark use, any other multiple of 16 is compiled at its first use
     ("attention_mfma", {"HD": 128}),
