@@ -540,6 +540,7 @@ extern "C" int qvl_gemm_resident(const void* x, int ldx, const void* h, int ldh,
   // that reads its rows again for every pass
   if (M <= 0 || N <= 0) return QVL_OK;
   if (M > 64) return QVL_ERR_LIMIT;
+  if (M > 32 && K > PASS_K) return QVL_ERR_LIMIT;   // teams of more than two keep their rows for a single pass
   if (K <= 0 || K % 8 || ldw % 8 || ldw < K || max_blocks <= 0 || !W || !out) return QVL_ERR_SHAPE;
   const bool norm = h != nullptr;
   const Plan pl = plan_for(M, K, norm, max_blocks, flags & 1);
@@ -602,6 +603,7 @@ extern "C" int qvl_gemm_resident_rope(const void* x, int ldx, const void* h, int
                                       int max_blocks, hipStream_t stream) {
   if (M <= 0) return QVL_OK;
   if (M > 64) return QVL_ERR_LIMIT;
+  if (M > 32 && K > PASS_K) return QVL_ERR_LIMIT;   // as in qvl_gemm_resident
   if (K <= 0 || K % 8 || ldw % 8 || ldw < K || max_blocks <= 0 || !W || !q_out) return QVL_ERR_SHAPE;
   if (nq <= 0 || nkv < 0 || hd <= 0 || hd % 16 || ps <= 0 || !cs) return QVL_ERR_SHAPE;
   if (nkv > 0 && (!slot || !kc || !vc)) return QVL_ERR_SHAPE;

@@ -70,8 +70,7 @@ def folds_norm(m: int, k: int, device=None) -> bool:
 def takes_resident(m: int, k: int, weight: torch.Tensor, *, norm: bool = False) -> bool:
     """Whether the resident kernel takes a product of ``m`` rows with this weight, and is the
     better choice for it.  A K that fits one pass of the block always is (the rows stay in
-    registers for all of the block's tiles), and so are 33 to 64 rows (teams of blocks with
-    resident rows).  Up to 32 rows with a longer K are read again for every pass of every tile,
+    registers for all of the block's tiles; with 33 to 64 rows in those of a team of blocks).  Up to 32 rows with a longer K are read again for every pass of every tile,
     which only pays while each compute unit has a single tile (at most 16 weight rows each):
     beyond that the library's product streams such a matrix faster (measured at the 72B
     decoder's shapes, K of 8192 and 29568)."""
@@ -79,7 +78,9 @@ def takes_resident(m: int, k: int, weight: torch.Tensor, *, norm: bool = False) 
         return False
     if norm:
         return folds_norm(m, k, weight.device)
-    if m > 32 or k <= (resident_norm_k() if m <= 16 else resident_two_tile_k()):
+    if m > 32:
+        return k <= resident_norm_k()    # teams keep their rows for one pass; in several passes they lose to the library
+    if k <= (resident_norm_k() if m <= 16 else resident_two_tile_k()):
         return True
     return weight.shape[0] <= 16 * _compute_units(weight.device)
 

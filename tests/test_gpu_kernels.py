@@ -286,8 +286,8 @@ def test_gemm_f32_is_exact_and_row_independent(m, n, k):
 def test_linear_bfloat16(m, n, k):
     """Up to 64 rows go through the resident matrix-core kernel (inner sizes in steps of 8): up to 32
     rows always if the inner size fits one pass of a block (4096, or 3840 with 17 to 32 rows), and
-    with a longer one while each compute unit has one tile at most; 33 to 64 rows always (their
-    rows are streamed); the rest through the library; all accumulate in float32."""
+    with a longer one while each compute unit has one tile at most; 33 to 64 rows if it fits one pass
+    (teams of blocks); the rest through the library; all accumulate in float32."""
     from qwen25vl_lite_amd.ops import skinny
     from qwen25vl_lite_amd.ops.linear import linear
     torch.manual_seed(k)
@@ -296,7 +296,7 @@ def test_linear_bfloat16(m, n, k):
     want = x.float() @ w.float().T
     units = torch.cuda.get_device_properties(0).multi_processor_count
     assert skinny.takes_resident(m, k, w.cuda()) == (
-        k % 8 == 0 and m <= 64 and (m > 32 or k <= (4096 if m <= 16 else 3840) or n <= 16 * units))
+        k % 8 == 0 and m <= 64 and (k <= 4096 if m > 32 else (k <= (4096 if m <= 16 else 3840) or n <= 16 * units)))
     out32 = linear(x.cuda(), w.cuda(), out_dtype=torch.float32)
     assert out32.dtype == torch.float32 and torch.allclose(out32.cpu(), want, atol=2e-3, rtol=2e-3)
     out16 = linear(x.cuda(), w.cuda())
@@ -307,6 +307,23 @@ def test_linear_bfloat16(m, n, k):
     if m > 1:
         alone = linear(x[m // 2:m // 2 + 1].contiguous().cuda(), w.cuda(), out_dtype=torch.float32)
         assert torch.allclose(alone[0], out32[m // 2], atol=1e-5, rtol=1e-5)
+
+
+@pytest.mark.parametrize("m, n, k", [(17, 300, 8200), (32, 3584, 18944), (25, 130, 4104)])
+def test_team_of_two_blocks_for_a_long_inner_size(m, n, k):
+    """17 to 32 rows whose inner size does not fit one pass: on request two blocks of one XCD walk
+    the same tiles, each with 16 of the rows (the kernel's other way is one block that reads its rows
+    again for every pass); both give the product."""
+    from qwen25vl_lite_amd.ops import skinny
+    torch.manual_seed(m)
+    x, w = torch.randn(m, k).bfloat16().cuda(), (torch.randn(n, k) / math.sqrt(k)).bfloat16().cuda()
+    want = x.float() @ w.float().T
+    team = skinny.resident_product(w, x=x, out_dtype=torch.float32, flags=skinny.TEAM_LONG_K)
+    assert torch.allclose(team, want, atol=2e-3, rtol=2e-3)
+    res = torch.randn(m, n).cuda()
+    into = res.clone()
+    skinny.resident_product(w, x=x, epilogue=skinny.RESIDUAL, out=into, flags=skinny.TEAM_LONG_K)
+    assert torch.allclose(into, res + want, atol=2e-3, rtol=2e-3)
 
 
 @pytest.mark.parametrize("m, n, k", [(1, 48, 64), (7, 1000, 3584), (16, 130, 4096), (3, 64, 144),
