@@ -60,13 +60,18 @@ __device__ __forceinline__ uint32_t pack2(float a, float b) {
 // of 16 lanes of its first operand with the even rows of its second, v_permlane32_swap the upper
 // half of the first with the lower half of the second: with both operands equal, the two results
 // hold each pair's two values in both lanes of the pair.
+__device__ __forceinline__ bf16x8_t ones8() {
+  const u32x4_t one = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
+  return __builtin_bit_cast(bf16x8_t, one);
+}
+__device__ __forceinline__ float max2(float a, float b);
 __device__ __forceinline__ float max_over_groups(float v) {
   const uint32_t b = __builtin_bit_cast(uint32_t, v);
   const auto x = __builtin_amdgcn_permlane16_swap(b, b, false, false);
-  v = fmaxf(__builtin_bit_cast(float, (uint32_t)x[0]), __builtin_bit_cast(float, (uint32_t)x[1]));
+  v = max2(__builtin_bit_cast(float, (uint32_t)x[0]), __builtin_bit_cast(float, (uint32_t)x[1]));
   const uint32_t c = __builtin_bit_cast(uint32_t, v);
   const auto y = __builtin_amdgcn_permlane32_swap(c, c, false, false);
-  return fmaxf(__builtin_bit_cast(float, (uint32_t)y[0]), __builtin_bit_cast(float, (uint32_t)y[1]));
+  return max2(__builtin_bit_cast(float, (uint32_t)y[0]), __builtin_bit_cast(float, (uint32_t)y[1]));
 }
 __device__ __forceinline__ float sum_over_groups(float v) {
   const uint32_t b = __builtin_bit_cast(uint32_t, v);
@@ -76,17 +81,18 @@ __device__ __forceinline__ float sum_over_groups(float v) {
   const auto y = __builtin_amdgcn_permlane32_swap(c, c, false, false);
   return __builtin_bit_cast(float, (uint32_t)y[0]) + __builtin_bit_cast(float, (uint32_t)y[1]);
 }
+// IEEE maximum (a NaN would come through; there is none): one v_maximum3_f32 for up to three values,
+// where fmaxf first makes each input canonical.
+__device__ __forceinline__ float max2(float a, float b) { return __builtin_elementwise_maximum(a, b); }
 
 // Softmax state of a column.  m is the reference the exponentials are taken against, in the
 // log2 domain (score * scale * log2 e).  It follows the running maximum lazily: it moves only
 // when a block's maximum exceeds it by more than LAZY_LOG2, so the sums are rarely rescaled and
-// no exponential exceeds 2^LAZY_LOG2; softmax does not depend on the reference.  l is this
-// lane's share of the column's sum (its 8 keys of every block); the four lanes of a column are
-// added up once, after the walk (total_sum).
+// no exponential exceeds 2^LAZY_LOG2; softmax does not depend on the reference.
 #define LAZY_LOG2 8.0f
 struct TileState {
-  float m, l;
-  f32x4_t acc[NT];
+  float m, l;            // l: this lane's share of the column's sum of probabilities (its 8 keys of every block), if the lanes add
+  f32x4_t acc[NT + 1];   // acc[NT]: the column's sum of probabilities in every row, if the matrix cores add (see Walk::compute)
 };
 
 // The page of each key row this lane loads in one 32-key block (two K row blocks, one V group).
@@ -141,6 +147,11 @@ struct Walk {
     for (int dt = 0; dt < NT; ++dt) rg.v[dt] = load8(vbase + (size_t)(dt * 16 + r) * ps);
   }
 
+  // BY_MATRIX: the way of the kernel for many tiles, whose waves are bound by the instructions they
+  // issue (the sum of the probabilities from the matrix cores, nothing done for a reference that
+  // stays); otherwise the way of the kernel for few tiles, which waits for memory and has no
+  // registers to spare.
+  template <bool BY_MATRIX>
   __device__ __forceinline__ void compute(int kb, const bf16x8_t (*qb)[KS], const BlockRegs& rg, TileState* sts) const {
     const int key0 = kb << 5;
     const bool interior = key0 >= all_lo && key0 + 31 <= all_hi;
@@ -172,39 +183,75 @@ struct Walk {
           raw[j] = ok ? raw[j] : -INFINITY;
         }
       }
-      float mloc = fmaxf(fmaxf(fmaxf(raw[0], raw[1]), fmaxf(raw[2], raw[3])),
-                         fmaxf(fmaxf(raw[4], raw[5]), fmaxf(raw[6], raw[7])));
-      mloc = max_over_groups(mloc) * scale_log2;   // scale_log2 > 0
-      const bool move = mloc > st.m + LAZY_LOG2;   // always at a column's first visible key (m = -inf)
-      const float m_new = move ? mloc : st.m;
-      const float alpha = move ? __builtin_amdgcn_exp2f(st.m - m_new) : 1.f;
-      // a column that has seen no key yet has m = -inf and only -inf scores: against 0 they give 0
-      const float ref = m_new == -INFINITY ? 0.f : m_new;
-      float psum = 0.f;
-      float pv[8];
+      // the largest of this lane's eight scores
+      float mloc = max2(max2(max2(raw[0], raw[1]), max2(raw[2], raw[3])),
+                        max2(max2(raw[4], raw[5]), max2(raw[6], raw[7]))) * scale_log2;   // scale_log2 > 0
+      if constexpr (!BY_MATRIX) {
+        mloc = max_over_groups(mloc);
+        const bool move = mloc > st.m + LAZY_LOG2;   // always at a column's first visible key (m = -inf)
+        const float m_new = move ? mloc : st.m;
+        const float alpha = move ? __builtin_amdgcn_exp2f(st.m - m_new) : 1.f;
+        // a column that has seen no key yet has m = -inf and only -inf scores: against 0 they give 0
+        const float ref = m_new == -INFINITY ? 0.f : m_new;
+        float psum = 0.f;
+        float pv[8];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        pv[j] = __builtin_amdgcn_exp2f(fmaf(raw[j], scale_log2, -ref));
-        psum += pv[j];
-      }
-      st.l = st.l * alpha + psum;
-      st.m = m_new;
-      // the reference rarely moves after the first blocks: skip the rescaling when no column of
-      // the wave needs it
-      const bool rescale = __any(move);
-      u32x4_t packed = {pack2(pv[0], pv[1]), pack2(pv[2], pv[3]), pack2(pv[4], pv[5]), pack2(pv[6], pv[7])};
-      const bf16x8_t pb = __builtin_bit_cast(bf16x8_t, packed);
-      if (rescale) {
-#pragma unroll
-        for (int dt = 0; dt < NT; ++dt) {
-          f32x4_t o = st.acc[dt];
-          o[0] *= alpha; o[1] *= alpha; o[2] *= alpha; o[3] *= alpha;
-          st.acc[dt] = o;
+        for (int j = 0; j < 8; ++j) {
+          pv[j] = __builtin_amdgcn_exp2f(fmaf(raw[j], scale_log2, -ref));
+          psum += pv[j];
         }
-      }
+        st.l = st.l * alpha + psum;
+        st.m = m_new;
+        // the reference rarely moves after the first blocks: skip the rescaling when no column of
+        // the wave needs it
+        const bool rescale = __any(move);
+        u32x4_t packed = {pack2(pv[0], pv[1]), pack2(pv[2], pv[3]), pack2(pv[4], pv[5]), pack2(pv[6], pv[7])};
+        const bf16x8_t pb = __builtin_bit_cast(bf16x8_t, packed);
+        if (rescale) {
 #pragma unroll
-      for (int dt = 0; dt < NT; ++dt)
-        st.acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(rg.v[dt], pb, st.acc[dt], 0, 0, 0);
+          for (int dt = 0; dt < NT; ++dt) {
+            f32x4_t o = st.acc[dt];
+            o[0] *= alpha; o[1] *= alpha; o[2] *= alpha; o[3] *= alpha;
+            st.acc[dt] = o;
+          }
+        }
+#pragma unroll
+        for (int dt = 0; dt < NT; ++dt)
+          st.acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(rg.v[dt], pb, st.acc[dt], 0, 0, 0);
+      } else {
+        // The column's four lanes hold the same m.  Only if one of them has a score far enough above
+        // it does the reference move (always at a column's first visible key, where m = -inf; rarely
+        // after a walk's first blocks), and only then do the lanes exchange their maxima and are
+        // the sums brought to the new reference.
+        if (__any(mloc > st.m + LAZY_LOG2)) {
+          mloc = max_over_groups(mloc);
+          const bool move = mloc > st.m + LAZY_LOG2;
+          const float m_new = move ? mloc : st.m;
+          const float alpha = move ? __builtin_amdgcn_exp2f(st.m - m_new) : 1.f;
+          st.m = m_new;
+#pragma unroll
+          for (int dt = 0; dt <= NT; ++dt) {
+            f32x4_t o = st.acc[dt];
+            o[0] *= alpha; o[1] *= alpha; o[2] *= alpha; o[3] *= alpha;
+            st.acc[dt] = o;
+          }
+        }
+        // a column that has seen no key yet has m = -inf and only -inf scores: against 0 they give 0.
+        // Inside the range that every column sees, every column has seen a key.
+        float nref = -st.m;
+        if (!interior) nref = st.m == -INFINITY ? 0.f : nref;
+        float pv[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) pv[j] = __builtin_amdgcn_exp2f(fmaf(raw[j], scale_log2, nref));
+        u32x4_t packed = {pack2(pv[0], pv[1]), pack2(pv[2], pv[3]), pack2(pv[4], pv[5]), pack2(pv[6], pv[7])};
+        const bf16x8_t pb = __builtin_bit_cast(bf16x8_t, packed);
+#pragma unroll
+        for (int dt = 0; dt < NT; ++dt)
+          st.acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(rg.v[dt], pb, st.acc[dt], 0, 0, 0);
+        // the sum of the probabilities comes from the matrix cores too: a row of ones beside the V^T
+        // rows adds up, for every column, exactly the rounded probabilities that the products use
+        st.acc[NT] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones8(), pb, st.acc[NT], 0, 0, 0);
+      }
     }
   }
 };
@@ -254,11 +301,11 @@ __device__ __forceinline__ void attend(const bf16_t* __restrict__ kc, const bf16
   for (;; kb += 2 * s) {
     if (LIVE(kb + 2 * s)) w.issue_pages(kb + 2 * s, p0);
     if (LIVE(kb + s)) w.issue_loads(kb + s, p1, rb);
-    w.compute(kb, qb, ra, st);
+    w.template compute<false>(kb, qb, ra, st);
     if (!LIVE(kb + s)) break;
     if (LIVE(kb + 3 * s)) w.issue_pages(kb + 3 * s, p1);
     if (LIVE(kb + 2 * s)) w.issue_loads(kb + 2 * s, p0, ra);
-    w.compute(kb + s, qb, rb, st);
+    w.template compute<false>(kb + s, qb, rb, st);
     if (!LIVE(kb + 2 * s)) break;
   }
 #undef LIVE
@@ -309,7 +356,7 @@ __device__ __forceinline__ void init_state(TileState& st) {
   st.m = -INFINITY;
   st.l = 0.f;
 #pragma unroll
-  for (int dt = 0; dt < NT; ++dt) st.acc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int dt = 0; dt <= NT; ++dt) st.acc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 }
 
 // ---- many tiles, keys shared through LDS -------------------------------------------------------
@@ -318,12 +365,19 @@ __device__ __forceinline__ void init_state(TileState& st) {
 // of its waves' key ranges.  Every 32-key block is fetched from the pages once per block, by all
 // waves together, and laid out in LDS the way the A operands want it, so the four waves share
 // every byte that leaves L2:
-//   K rows in the permuted order of the top of the file (row 16 b + r holds the key of K block b,
-//   row r), each row padded by 16 bytes: the 16 lanes of a row group read 16 different banks;
-//   V^T rows of 32 keys padded to 40: a stride of 5 x 16 bytes is coprime with the 16 bank groups.
+//   K rows by key, each padded by 16 bytes, the second 16 keys beginning at row K_HALF_ROW = 20: the
+//   16 lanes of a row group (keys 4b .. 4b+3 and 4b+8 .. 4b+11 of either half, see the top of the
+//   file) then read 16 different bank groups;
+//   V^T as two arrays [channel][2 chunks of 8 keys], one for each half of the block's keys, the two
+//   chunks of channels 8 .. 15 (mod 16) swapped: no padding, and again 16 different bank groups.
 // The data goes from global memory straight into LDS (global_load_lds_dwordx4: lane l of a wave
 // puts its 16 bytes at M0 + 16 l, so one instruction fills 1 KB of a stage and each lane works out
-// which 16 bytes of the pages belong there; lanes on padding fetch a neighbour's bytes again).
+// once per walk which 16 bytes of a page belong there; lanes on padding fetch a neighbour's bytes
+// again).  The two halves of a block's keys may lie in different pages.  The layout keeps them
+// apart, so that nearly every load instruction reads one page only: its address is a scalar base,
+// worked out once per block and half, plus the lane's constant offset, and issuing a block's loads
+// costs a wave a few scalar instructions.  (A wave has two in flight on its SIMD at best and
+// issues an instruction every eight cycles or so: every instruction of the loop counts, whatever unit runs it.)
 // No register holds data in flight, so BLK_STAGES - 1 blocks are on their way while one is
 // computed.  The loads are issued from inline assembly and waited for with explicit vmcnt values:
 // every wave issues exactly WAVE_LOADS of them per block.
@@ -345,9 +399,11 @@ __device__ __forceinline__ void init_state(TileState& st) {
 #define BLK_STAGES 4
 #define CH_PER_KEY (HD / 8)                                       // 16-byte chunks of a key
 #define KROW (HD + 8)                                             // elements of a K row in LDS
-#define VROW 40
-#define K_LOADS ((32 * (CH_PER_KEY + 1) + 63) / 64)               // 1 KB wave loads that cover the K rows
-#define V_LOADS ((HD * 5 + 63) / 64)
+#define K_HALF_ROW 20                                             // the row of the second half's first key
+#define K_SLOTS ((K_HALF_ROW + 16) * (CH_PER_KEY + 1))            // 16-byte slots of the K rows
+#define K_LOADS ((K_SLOTS + 63) / 64)                             // 1 KB wave loads that cover them
+#define V_HALF_SLOTS ((2 * HD + 63) / 64 * 64)                    // slots of one half of the V^T rows (whole loads)
+#define V_LOADS (2 * V_HALF_SLOTS / 64)
 #define STAGE_LOADS (K_LOADS + V_LOADS)
 #define WAVE_LOADS ((STAGE_LOADS + BLK_WAVES - 1) / BLK_WAVES)
 #define STAGE_ELEMS (STAGE_LOADS * 512)
@@ -357,6 +413,10 @@ __device__ __forceinline__ void init_state(TileState& st) {
 
 __device__ __forceinline__ void load16_to_lds(const bf16_t* g, uint32_t lds_byte_address) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds_byte_address) : "memory");
+}
+// The same with the address as a base that all lanes share (scalar registers) plus a lane's byte offset.
+__device__ __forceinline__ void load16_to_lds(const bf16_t* base, uint32_t lane_bytes, uint32_t lds_byte_address) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_bytes), "s"(base), "s"(lds_byte_address) : "memory");
 }
 // Wait until at most n of this wave's loads are outstanding (they finish in order).
 template <int N>
@@ -371,72 +431,96 @@ struct StagePages {
   int page[2], off[2];
 };
 
+// Which half of the block's keys load t of a stage reads: 0 or 1, or 2 if its lanes differ.
+// Loads 0 .. K_LOADS - 1 fill the K rows (slot q is chunk q mod (CH_PER_KEY + 1) of row
+// q / (CH_PER_KEY + 1); rows 16 .. K_HALF_ROW - 1 hold nothing), the others the V^T rows (slot q
+// of a half is chunk q mod 2 of channel q / 2).
+__host__ __device__ constexpr int load_half(int t) {
+  if (t >= K_LOADS) return (t - K_LOADS) * 64 / V_HALF_SLOTS;
+  const int last_slot = 64 * t + 63 < K_SLOTS - 1 ? 64 * t + 63 : K_SLOTS - 1;
+  const bool first_half = 64 * t / (CH_PER_KEY + 1) < 16, second_half = last_slot / (CH_PER_KEY + 1) >= K_HALF_ROW;
+  return first_half && second_half ? 2 : (second_half ? 1 : 0);
+}
+
 // Wave w issues the loads t = (w + BLK_WAVES i) mod STAGE_LOADS, i < WAVE_LOADS, of a block (a
-// load may be issued twice: same bytes to the same place).  Load t < K_LOADS fills K slots
-// 64 t .. 64 t + 63, the others V slots; slot q of K is chunk q mod (CH_PER_KEY + 1) of row
-// q / (CH_PER_KEY + 1), slot q of V^T is keys 8 (q mod 5) .. + 7 of channel q / 5.  Everything
-// about a lane's address that does not change from block to block is worked out once (start);
-// the halves' page index and slot move along with the blocks (next_pages is called for
-// the blocks kb, kb + GROUPS, ... of a group), so the page size is divided by once.
+// load may be issued twice: same bytes to the same place).  Everything about a lane's address that
+// does not change from block to block is worked out once (start); the halves' page index and slot
+// move along with the blocks (next_pages is called for the blocks kb, kb + GROUPS, ... of a
+// group), so the page size is divided by once.
 template <int GROUPS>
 struct BlockLoader {
-  const bf16_t* kc;
-  const bf16_t* vc;
+  const bf16_t* kbase;           // the head's first key in page 0, and its first value
+  const bf16_t* vbase;
   const int* bt;
   int table_width, ps, wave;
   size_t page_stride;            // elements of one page over all heads, K and V alike
-  int idx[2], off[2];            // of the next block's halves
-  int fixed[WAVE_LOADS];         // element offset of the lane's bytes in the page when its half begins at slot 0
-  uint32_t halves;               // bit i: load i takes the second half's page
+  int idx, off;                  // page index and slot of the next block's first half (its second half begins 16 keys on)
+  int step_pages, step_slots;    // from one block of the group to its next: whole pages and slots
+  uint32_t fixed[WAVE_LOADS];    // byte offset of the lane's 16 bytes from where its half begins in its page
+  uint32_t halves;               // bit i: the lane's bytes of load i belong to the second half (loads of both halves only)
 
-  __device__ __forceinline__ int load_index(int i) const { return (wave + BLK_WAVES * i) % STAGE_LOADS; }
-
-  __device__ __forceinline__ void start(int kb, int nkv, int kvh) {
+  __device__ __forceinline__ void start(const bf16_t* kc, const bf16_t* vc, int kb, int nkv, int kvh) {
     const int lane = threadIdx.x & 63;
     page_stride = (size_t)nkv * ps * HD;
+    kbase = kc + (size_t)kvh * ps * HD;
+    vbase = vc + (size_t)kvh * HD * ps;
     halves = 0;
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const int key = (kb << 5) + 16 * h;
-      idx[h] = key / ps;
-      off[h] = key - idx[h] * ps;
-    }
+    idx = (kb << 5) / ps;
+    off = (kb << 5) - idx * ps;
+    step_pages = 32 * GROUPS / ps;
+    step_slots = 32 * GROUPS - step_pages * ps;
 #pragma unroll
     for (int i = 0; i < WAVE_LOADS; ++i) {
-      const int t = load_index(i);
+      const int t = (wave + BLK_WAVES * i) % STAGE_LOADS;
       if (t < K_LOADS) {
-        const int slot = 64 * t + lane;
+        int slot = 64 * t + lane;
+        slot = slot < K_SLOTS ? slot : K_SLOTS - 1;
         int row = slot / (CH_PER_KEY + 1), part = slot - row * (CH_PER_KEY + 1);
-        row = row < 32 ? row : 31;
         part = part < CH_PER_KEY ? part : CH_PER_KEY - 1;
-        const int b = row >> 4, r = row & 15;
-        const int kk = 8 * (r >> 2) + 4 * b + (r & 3);   // the key of LDS row 16 b + r
-        halves |= (kk >= 16 ? 1u : 0u) << i;
-        fixed[i] = (kvh * ps + (kk & 15)) * HD + part * 8;
+        // a row that holds nothing reads what the load's other lanes read (a load of both halves: the first)
+        const int half = row >= K_HALF_ROW ? 1 : (row < 16 ? 0 : (load_half(t) == 1 ? 1 : 0));
+        const int key = row >= K_HALF_ROW ? row - K_HALF_ROW : (row < 16 ? row : 0);
+        halves |= (uint32_t)half << i;
+        fixed[i] = 2u * (uint32_t)(key * HD + part * 8);
       } else {
-        const int slot = 64 * (t - K_LOADS) + lane;
-        int row = slot / 5, part = slot - row * 5;
+        const int slot = (64 * (t - K_LOADS) + lane) % V_HALF_SLOTS;
+        int row = slot >> 1;
         row = row < HD ? row : HD - 1;
-        part = part < 4 ? part : 3;
-        halves |= (part >= 2 ? 1u : 0u) << i;
-        fixed[i] = (kvh * HD + row) * ps + 8 * (part & 1);
+        const int chunk = (slot & 1) ^ ((row >> 3) & 1);
+        fixed[i] = 2u * (uint32_t)(row * ps + 8 * chunk);
       }
     }
   }
   // Pages of the next block; keys past the table or without a page (nobody sees them) read page 0.
+  // The table entries are only asked for here: waiting for them is left to issue(), a block's work later.
   __device__ __forceinline__ void next_pages(StagePages& pg) {
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const int p = idx[h] < table_width ? bt[idx[h]] : 0;
-      pg.page[h] = p < 0 ? 0 : p;
-      pg.off[h] = off[h];
-      off[h] += 32 * GROUPS;  // the group's next block; a page has at least 16 slots
-#pragma unroll
-      for (int i = 0; i < 2 * GROUPS; ++i)
-        if (off[h] >= ps) {
-          off[h] -= ps;
-          ++idx[h];
-        }
+    const bool same = off + 16 < ps;   // both halves in one page
+    const int idx1 = same ? idx : idx + 1;
+    pg.page[0] = idx < table_width ? bt[idx] : 0;   // as the table has it
+    pg.page[1] = idx1 < table_width ? bt[idx1] : 0;
+    pg.off[0] = off;
+    pg.off[1] = same ? off + 16 : 0;
+    idx += step_pages;
+    off += step_slots;
+    if (off >= ps) {
+      off -= ps;
+      ++idx;
+    }
+  }
+  // Load I of wave W: which load of the stage it is, whether it reads keys or values and from which
+  // half's page are known when the kernel is compiled.
+  template <int W, int I>
+  __device__ __forceinline__ void issue_from(const bf16_t* const* kh, const bf16_t* const* vh, uint32_t stage) const {
+    if constexpr (I < WAVE_LOADS) {
+      constexpr int t = (W + BLK_WAVES * I) % STAGE_LOADS, half = load_half(t);
+      const uint32_t lds = stage + 1024u * t;
+      if constexpr (half < 2) {
+        load16_to_lds(t < K_LOADS ? kh[half] : vh[half], fixed[I], lds);
+      } else {
+        const bf16_t* base = ((halves >> I) & 1u) ? kh[1] : kh[0];   // only K loads read both halves
+        load16_to_lds(reinterpret_cast<const bf16_t*>(reinterpret_cast<const char*>(base) + fixed[I]), lds);
+      }
+      issue_from<W, I + 1>(kh, vh, stage);
     }
   }
   // Issue this wave's loads of the block with pages pg into the stage at LDS byte address stage.
@@ -446,35 +530,34 @@ struct BlockLoader {
     const bf16_t* vh[2];
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-      kh[h] = kc + (size_t)pg.page[h] * page_stride + pg.off[h] * HD;
-      vh[h] = vc + (size_t)pg.page[h] * page_stride + pg.off[h];
+      const size_t page = (size_t)(pg.page[h] < 0 ? 0 : pg.page[h]) * page_stride;
+      kh[h] = kbase + page + (uint32_t)pg.off[h] * (uint32_t)HD;
+      vh[h] = vbase + page + (uint32_t)pg.off[h];
     }
-#pragma unroll
-    for (int i = 0; i < WAVE_LOADS; ++i) {
-      const int t = load_index(i);
-      const bool second = (halves >> i) & 1u;
-      // keys or values is the same for the whole wave: chosen in scalar registers, before the lanes
-      // choose their half
-      const bool keys = t < K_LOADS;
-      const bf16_t* first_half = keys ? kh[0] : vh[0];
-      const bf16_t* second_half = keys ? kh[1] : vh[1];
-      const bf16_t* base = second ? second_half : first_half;
-      load16_to_lds(base + fixed[i], __builtin_amdgcn_readfirstlane(stage + 1024u * t));
-    }
+    if (wave == 0) issue_from<0, 0>(kh, vh, stage);
+    else if (wave == 1) issue_from<1, 0>(kh, vh, stage);
+    else if (wave == 2) issue_from<2, 0>(kh, vh, stage);
+    else issue_from<3, 0>(kh, vh, stage);
   }
 };
+static_assert(BLK_WAVES == 4, "issue() names the waves");
 
 __device__ __forceinline__ void operands_from_lds(const bf16_t* ks, const bf16_t* vs, BlockRegs& rg) {
   const int lane = threadIdx.x & 63, lg = lane >> 4, r = lane & 15;
+  // row r of K block b holds key 8 (r / 4) + 4 b + r % 4 of the block's 32 (see the top of the file)
 #pragma unroll
-  for (int b = 0; b < 2; ++b)
+  for (int b = 0; b < 2; ++b) {
+    const int row = (r >> 3) * K_HALF_ROW + 8 * ((r >> 2) & 1) + 4 * b + (r & 3);
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
       const int d = s * 32 + 8 * lg;
-      rg.k[b][s] = (d < HD) ? load8(ks + (16 * b + r) * KROW + d) : zero8();
+      rg.k[b][s] = (d < HD) ? load8(ks + row * KROW + d) : zero8();
     }
+  }
+  // keys 8 lg .. 8 lg + 7 of channel dt * 16 + r: half lg / 2, chunk lg % 2, swapped for channels 8 .. 15
+  const int vslot = (lg >> 1) * V_HALF_SLOTS + 2 * r + ((lg & 1) ^ (r >> 3));
 #pragma unroll
-  for (int dt = 0; dt < NT; ++dt) rg.v[dt] = load8(vs + (dt * 16 + r) * VROW + 8 * lg);
+  for (int dt = 0; dt < NT; ++dt) rg.v[dt] = load8(vs + (vslot + 32 * dt) * 8);
 }
 
 // One entry of the block list for one key/value head.  blk_cb counts in units of
@@ -555,7 +638,7 @@ __device__ __forceinline__ void attend_block(BlockShared<GROUPS>& sh, int item, 
     w.all_hi = b;
   }
   BlockLoader<GROUPS> ld;
-  ld.kc = kc; ld.vc = vc; ld.bt = bt + (size_t)r * table_width;
+  ld.bt = bt + (size_t)r * table_width;
   ld.table_width = table_width; ld.ps = ps; ld.wave = wave;
   // this group's blocks are kb0, kb0 + GROUPS, ...: nblk of them; every group goes round the
   // loop (and through its barrier) as often as the first
@@ -564,7 +647,7 @@ __device__ __forceinline__ void attend_block(BlockShared<GROUPS>& sh, int item, 
   const int rounds = (all_blocks + GROUPS - 1) / GROUPS;
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)&sh.stage[group][0][0];
   StagePages pg;
-  ld.start(kb0, nkv, kvh);
+  ld.start(kc, vc, kb0, nkv, kvh);
   ld.next_pages(pg);
   // the queries are in their registers before the first asynchronous load is issued: from here to
   // the end of the walk the compiler finds nothing of its own to wait for in vmcnt
@@ -594,7 +677,7 @@ __device__ __forceinline__ void attend_block(BlockShared<GROUPS>& sh, int item, 
       const bf16_t* stage = sh.stage[group][i % BLK_STAGES];
       BlockRegs ops;
       operands_from_lds(stage, stage + K_LOADS * 512, ops);
-      w.compute(kb, qb, ops, st);
+      w.template compute<true>(kb, qb, ops, st);
     }
   }
   if (GROUPS > 1) {
@@ -611,7 +694,7 @@ __device__ __forceinline__ void attend_block(BlockShared<GROUPS>& sh, int item, 
 #pragma unroll
           for (int j = 0; j < 4; ++j) mine[(dt * 4 + j) * BLK_WAVES * 64] = st[i].acc[dt][j];
         mine[(NT * 4) * BLK_WAVES * 64] = st[i].m;
-        mine[(NT * 4 + 1) * BLK_WAVES * 64] = st[i].l;
+        mine[(NT * 4 + 1) * BLK_WAVES * 64] = st[i].acc[NT][0];
       }
     }
     __syncthreads();
@@ -623,7 +706,7 @@ __device__ __forceinline__ void attend_block(BlockShared<GROUPS>& sh, int item, 
       const float m = fmaxf(st[i].m, m_b);
       const float ref = m == -INFINITY ? 0.f : m;   // a column without keys: both sides are zero
       const float sa = __builtin_amdgcn_exp2f(st[i].m - ref), sb = __builtin_amdgcn_exp2f(m_b - ref);
-      st[i].l = st[i].l * sa + l_b * sb;
+      st[i].acc[NT][0] = st[i].acc[NT][0] * sa + l_b * sb;
 #pragma unroll
       for (int dt = 0; dt < NT; ++dt)
 #pragma unroll
@@ -634,7 +717,7 @@ __device__ __forceinline__ void attend_block(BlockShared<GROUPS>& sh, int item, 
   const int lg = lane >> 4;
 #pragma unroll
   for (int i = 0; i < BLK_CT; ++i) {
-    const float total = sum_over_groups(st[i].l);
+    const float total = st[i].acc[NT][0];
     if (!t[i].valid) continue;
     const float inv = 1.0f / total;
     bf16_t* orow = out + ((size_t)t[i].token * nq + t[i].head) * HD;
