@@ -23,6 +23,7 @@
 // registers, and merge through LDS; for very long contexts the keys are further split among
 // blocks, whose partial sums a second kernel merges.
 #include "common.h"
+#include <type_traits>
 #include "attention_mfma.h"
 #include <mutex>
 
@@ -365,19 +366,21 @@ __device__ __forceinline__ void init_state(TileState& st) {
 // of its waves' key ranges.  Every 32-key block is fetched from the pages once per block, by all
 // waves together, and laid out in LDS the way the A operands want it, so the four waves share
 // every byte that leaves L2:
-//   K rows by key, each padded by 16 bytes, the second 16 keys beginning at row K_HALF_ROW = 20: the
-//   16 lanes of a row group (keys 4b .. 4b+3 and 4b+8 .. 4b+11 of either half, see the top of the
-//   file) then read 16 different bank groups;
+//   K rows by key, each padded by 16 bytes, the two halves of the block's keys in regions of whole
+//   1 KB loads, the second half's rows set off by K_SKEW slots: the 16 lanes of a row group (keys
+//   4b .. 4b+3 and 4b+8 .. 4b+11 of either half, see the top of the file) then read 16 different
+//   bank groups when the head size is a multiple of 128;
 //   V^T as two arrays [channel][2 chunks of 8 keys], one for each half of the block's keys, the two
 //   chunks of channels 8 .. 15 (mod 16) swapped: no padding, and again 16 different bank groups.
 // The data goes from global memory straight into LDS (global_load_lds_dwordx4: lane l of a wave
 // puts its 16 bytes at M0 + 16 l, so one instruction fills 1 KB of a stage and each lane works out
 // once per walk which 16 bytes of a page belong there; lanes on padding fetch a neighbour's bytes
-// again).  The two halves of a block's keys may lie in different pages.  The layout keeps them
-// apart, so that nearly every load instruction reads one page only: its address is a scalar base,
-// worked out once per block and half, plus the lane's constant offset, and issuing a block's loads
-// costs a wave a few scalar instructions.  (A wave has two in flight on its SIMD at best and
-// issues an instruction every eight cycles or so: every instruction of the loop counts, whatever unit runs it.)
+// again).  The two halves of a block's keys may lie in different pages, and a stage has four parts:
+// the K rows and the V^T rows of either half.  Each of the four waves fills one part, so all that
+// a wave does for a block's loads is one table lookup, one base address (scalar arithmetic) and a
+// few load instructions with that base and the lanes' constant offsets.  (A wave issues an
+// instruction every eight clocks or so and a SIMD holds two of these waves: every instruction of
+// the loop counts, whatever unit runs it.)
 // No register holds data in flight, so BLK_STAGES - 1 blocks are on their way while one is
 // computed.  The loads are issued from inline assembly and waited for with explicit vmcnt values:
 // every wave issues exactly WAVE_LOADS of them per block.
@@ -399,24 +402,22 @@ __device__ __forceinline__ void init_state(TileState& st) {
 #define BLK_STAGES 4
 #define CH_PER_KEY (HD / 8)                                       // 16-byte chunks of a key
 #define KROW (HD + 8)                                             // elements of a K row in LDS
-#define K_HALF_ROW 20                                             // the row of the second half's first key
-#define K_SLOTS ((K_HALF_ROW + 16) * (CH_PER_KEY + 1))            // 16-byte slots of the K rows
-#define K_LOADS ((K_SLOTS + 63) / 64)                             // 1 KB wave loads that cover them
+#define K_SKEW ((4 * (CH_PER_KEY + 1)) % 16)                      // 16-byte slots by which the second half's rows are set off
+#define KH_LOADS ((16 * (CH_PER_KEY + 1) + K_SKEW + 63) / 64)     // 1 KB wave loads that cover the K rows of one half
+#define K_LOADS (2 * KH_LOADS)
 #define V_HALF_SLOTS ((2 * HD + 63) / 64 * 64)                    // slots of one half of the V^T rows (whole loads)
-#define V_LOADS (2 * V_HALF_SLOTS / 64)
+#define VH_LOADS (V_HALF_SLOTS / 64)
+#define V_LOADS (2 * VH_LOADS)
 #define STAGE_LOADS (K_LOADS + V_LOADS)
-#define WAVE_LOADS ((STAGE_LOADS + BLK_WAVES - 1) / BLK_WAVES)
+#define WAVE_LOADS (KH_LOADS > VH_LOADS ? KH_LOADS : VH_LOADS)    // what a wave issues a block: one of the four parts of a stage
 #define STAGE_ELEMS (STAGE_LOADS * 512)
 #if 2 * WAVE_LOADS > 63
 #error "the in-flight loads of a wave do not fit the vmcnt counter"
 #endif
 
-__device__ __forceinline__ void load16_to_lds(const bf16_t* g, uint32_t lds_byte_address) {
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds_byte_address) : "memory");
-}
-// The same with the address as a base that all lanes share (scalar registers) plus a lane's byte offset.
-__device__ __forceinline__ void load16_to_lds(const bf16_t* base, uint32_t lane_bytes, uint32_t lds_byte_address) {
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_bytes), "s"(base), "s"(lds_byte_address) : "memory");
+// The LDS address is stage + offset: added straight into M0.
+__device__ __forceinline__ void load16_to_lds(const char* base, uint32_t lane_bytes, uint32_t stage, uint32_t offset) {
+  asm volatile("s_add_i32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_bytes), "s"(base), "s"(stage), "s"(offset) : "memory", "scc");
 }
 // Wait until at most n of this wave's loads are outstanding (they finish in order).
 template <int N>
@@ -424,82 +425,72 @@ __device__ __forceinline__ void wait_loads() {
   __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0f70);
 }
 
-// The pages of the two 16-key halves of a block and the slot in the page where each half begins
-// (a page holds a multiple of 16 keys, so a half never straddles pages).  The same for every
-// thread: the compiler keeps these in scalar registers and fetches the table entries once per wave.
+// The page of the 16-key half of a block that a wave loads from, as the block table has it, and
+// the slot in the page where the half begins (a page holds a multiple of 16 keys, so a half never
+// straddles pages).  The same for every thread of the wave: scalar registers.
 struct StagePages {
-  int page[2], off[2];
+  int page, off;
 };
 
-// Which half of the block's keys load t of a stage reads: 0 or 1, or 2 if its lanes differ.
-// Loads 0 .. K_LOADS - 1 fill the K rows (slot q is chunk q mod (CH_PER_KEY + 1) of row
-// q / (CH_PER_KEY + 1); rows 16 .. K_HALF_ROW - 1 hold nothing), the others the V^T rows (slot q
-// of a half is chunk q mod 2 of channel q / 2).
-__host__ __device__ constexpr int load_half(int t) {
-  if (t >= K_LOADS) return (t - K_LOADS) * 64 / V_HALF_SLOTS;
-  const int last_slot = 64 * t + 63 < K_SLOTS - 1 ? 64 * t + 63 : K_SLOTS - 1;
-  const bool first_half = 64 * t / (CH_PER_KEY + 1) < 16, second_half = last_slot / (CH_PER_KEY + 1) >= K_HALF_ROW;
-  return first_half && second_half ? 2 : (second_half ? 1 : 0);
-}
-
-// Wave w issues the loads t = (w + BLK_WAVES i) mod STAGE_LOADS, i < WAVE_LOADS, of a block (a
-// load may be issued twice: same bytes to the same place).  Everything about a lane's address that
-// does not change from block to block is worked out once (start); the halves' page index and slot
-// move along with the blocks (next_pages is called for the blocks kb, kb + GROUPS, ... of a
+// Wave w of a group fills part w of a stage: the K rows (w < 2) or V^T rows of half w % 2 of the
+// block's keys, with WAVE_LOADS loads (a part with fewer issues its last again: same bytes to the
+// same place, and every wave has the same number in flight).  Everything about a lane's address
+// that does not change from block to block is worked out once (start); the half's page index and
+// slot move along with the blocks (next_pages is called for the blocks kb, kb + GROUPS, ... of a
 // group), so the page size is divided by once.
 template <int GROUPS>
 struct BlockLoader {
-  const bf16_t* kbase;           // the head's first key in page 0, and its first value
-  const bf16_t* vbase;
+  const char* base;              // of the head's keys (or values) in page 0
   const int* bt;
   int table_width, ps, wave;
-  size_t page_stride;            // elements of one page over all heads, K and V alike
-  int idx, off;                  // page index and slot of the next block's first half (its second half begins 16 keys on)
+  uint32_t page_bytes;           // bytes of one page over all heads, K and V alike
+  uint32_t slot_bytes;           // bytes from one slot of a page to the next: a key's HD values, or one value of a V^T row
+  int idx, off;                  // page index and slot of the half in the next block
   int step_pages, step_slots;    // from one block of the group to its next: whole pages and slots
-  uint32_t fixed[WAVE_LOADS];    // byte offset of the lane's 16 bytes from where its half begins in its page
-  uint32_t halves;               // bit i: the lane's bytes of load i belong to the second half (loads of both halves only)
+  uint32_t part_offset[WAVE_LOADS];   // of the load's 1 KB in a stage
+  uint32_t fixed[WAVE_LOADS];    // byte offset of the lane's 16 bytes from where the half begins in its page
 
   __device__ __forceinline__ void start(const bf16_t* kc, const bf16_t* vc, int kb, int nkv, int kvh) {
     const int lane = threadIdx.x & 63;
-    page_stride = (size_t)nkv * ps * HD;
-    kbase = kc + (size_t)kvh * ps * HD;
-    vbase = vc + (size_t)kvh * HD * ps;
-    halves = 0;
-    idx = (kb << 5) / ps;
-    off = (kb << 5) - idx * ps;
+    const bool keys = wave < 2;
+    const int half = wave & 1;
+    page_bytes = 2u * (uint32_t)nkv * (uint32_t)ps * (uint32_t)HD;
+    slot_bytes = keys ? 2u * HD : 2u;
+    base = keys ? reinterpret_cast<const char*>(kc + (size_t)kvh * ps * HD) : reinterpret_cast<const char*>(vc + (size_t)kvh * HD * ps);
+    const int key = (kb << 5) + 16 * half;
+    idx = key / ps;
+    off = key - idx * ps;
     step_pages = 32 * GROUPS / ps;
     step_slots = 32 * GROUPS - step_pages * ps;
 #pragma unroll
     for (int i = 0; i < WAVE_LOADS; ++i) {
-      const int t = (wave + BLK_WAVES * i) % STAGE_LOADS;
-      if (t < K_LOADS) {
-        int slot = 64 * t + lane;
-        slot = slot < K_SLOTS ? slot : K_SLOTS - 1;
+      if (keys) {
+        const int load = i < KH_LOADS ? i : KH_LOADS - 1;
+        part_offset[i] = 1024u * (uint32_t)(half * KH_LOADS + load);
+        int slot = 64 * load + lane - half * K_SKEW;   // of the half's rows
+        slot = slot < 0 ? 0 : slot;
         int row = slot / (CH_PER_KEY + 1), part = slot - row * (CH_PER_KEY + 1);
+        row = row < 16 ? row : 15;
         part = part < CH_PER_KEY ? part : CH_PER_KEY - 1;
-        // a row that holds nothing reads what the load's other lanes read (a load of both halves: the first)
-        const int half = row >= K_HALF_ROW ? 1 : (row < 16 ? 0 : (load_half(t) == 1 ? 1 : 0));
-        const int key = row >= K_HALF_ROW ? row - K_HALF_ROW : (row < 16 ? row : 0);
-        halves |= (uint32_t)half << i;
-        fixed[i] = 2u * (uint32_t)(key * HD + part * 8);
+        fixed[i] = 2u * (uint32_t)(row * HD + part * 8);
       } else {
-        const int slot = (64 * (t - K_LOADS) + lane) % V_HALF_SLOTS;
+        const int load = i < VH_LOADS ? i : VH_LOADS - 1;
+        part_offset[i] = 1024u * (uint32_t)(K_LOADS + half * VH_LOADS + load);
+        const int slot = 64 * load + lane;
         int row = slot >> 1;
         row = row < HD ? row : HD - 1;
         const int chunk = (slot & 1) ^ ((row >> 3) & 1);
         fixed[i] = 2u * (uint32_t)(row * ps + 8 * chunk);
       }
     }
+#pragma unroll
+    for (int i = 0; i < WAVE_LOADS; ++i) part_offset[i] = __builtin_amdgcn_readfirstlane(part_offset[i]);
   }
-  // Pages of the next block; keys past the table or without a page (nobody sees them) read page 0.
-  // The table entries are only asked for here: waiting for them is left to issue(), a block's work later.
+  // The half's page in the next block; keys past the table or without a page (nobody sees them) read
+  // page 0.  The table entry is only asked for here: waiting for it is left to issue(), a block's work later.
   __device__ __forceinline__ void next_pages(StagePages& pg) {
-    const bool same = off + 16 < ps;   // both halves in one page
-    const int idx1 = same ? idx : idx + 1;
-    pg.page[0] = idx < table_width ? bt[idx] : 0;   // as the table has it
-    pg.page[1] = idx1 < table_width ? bt[idx1] : 0;
-    pg.off[0] = off;
-    pg.off[1] = same ? off + 16 : 0;
+    pg.page = idx < table_width ? bt[idx] : 0;   // as the table has it
+    pg.off = off;
     idx += step_pages;
     off += step_slots;
     if (off >= ps) {
@@ -507,51 +498,26 @@ struct BlockLoader {
       ++idx;
     }
   }
-  // Load I of wave W: which load of the stage it is, whether it reads keys or values and from which
-  // half's page are known when the kernel is compiled.
-  template <int W, int I>
-  __device__ __forceinline__ void issue_from(const bf16_t* const* kh, const bf16_t* const* vh, uint32_t stage) const {
-    if constexpr (I < WAVE_LOADS) {
-      constexpr int t = (W + BLK_WAVES * I) % STAGE_LOADS, half = load_half(t);
-      const uint32_t lds = stage + 1024u * t;
-      if constexpr (half < 2) {
-        load16_to_lds(t < K_LOADS ? kh[half] : vh[half], fixed[I], lds);
-      } else {
-        const bf16_t* base = ((halves >> I) & 1u) ? kh[1] : kh[0];   // only K loads read both halves
-        load16_to_lds(reinterpret_cast<const bf16_t*>(reinterpret_cast<const char*>(base) + fixed[I]), lds);
-      }
-      issue_from<W, I + 1>(kh, vh, stage);
-    }
-  }
-  // Issue this wave's loads of the block with pages pg into the stage at LDS byte address stage.
+  // Issue this wave's loads of the block with page pg into the stage at LDS byte address stage.
   __device__ __forceinline__ void issue(const StagePages& pg, uint32_t stage) const {
-    // where each half begins, for K and for V: the same for all threads (scalar arithmetic)
-    const bf16_t* kh[2];
-    const bf16_t* vh[2];
+    const char* from = base + (uint64_t)(uint32_t)(pg.page < 0 ? 0 : pg.page) * page_bytes + (uint32_t)pg.off * slot_bytes;
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const size_t page = (size_t)(pg.page[h] < 0 ? 0 : pg.page[h]) * page_stride;
-      kh[h] = kbase + page + (uint32_t)pg.off[h] * (uint32_t)HD;
-      vh[h] = vbase + page + (uint32_t)pg.off[h];
-    }
-    if (wave == 0) issue_from<0, 0>(kh, vh, stage);
-    else if (wave == 1) issue_from<1, 0>(kh, vh, stage);
-    else if (wave == 2) issue_from<2, 0>(kh, vh, stage);
-    else issue_from<3, 0>(kh, vh, stage);
+    for (int i = 0; i < WAVE_LOADS; ++i) load16_to_lds(from, fixed[i], stage, part_offset[i]);
   }
 };
-static_assert(BLK_WAVES == 4, "issue() names the waves");
+static_assert(BLK_WAVES == 4, "a stage has four parts, one a wave");
 
 __device__ __forceinline__ void operands_from_lds(const bf16_t* ks, const bf16_t* vs, BlockRegs& rg) {
   const int lane = threadIdx.x & 63, lg = lane >> 4, r = lane & 15;
-  // row r of K block b holds key 8 (r / 4) + 4 b + r % 4 of the block's 32 (see the top of the file)
+  // row r of K block b holds key 8 (r / 4) + 4 b + r % 4 of the block's 32 (see the top of the file):
+  // key 8 (r / 4 % 2) + 4 b + r % 4 of half r / 8
 #pragma unroll
   for (int b = 0; b < 2; ++b) {
-    const int row = (r >> 3) * K_HALF_ROW + 8 * ((r >> 2) & 1) + 4 * b + (r & 3);
+    const bf16_t* row = ks + (r >> 3) * (KH_LOADS * 512 + K_SKEW * 8) + (8 * ((r >> 2) & 1) + 4 * b + (r & 3)) * KROW;
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
       const int d = s * 32 + 8 * lg;
-      rg.k[b][s] = (d < HD) ? load8(ks + row * KROW + d) : zero8();
+      rg.k[b][s] = (d < HD) ? load8(row + d) : zero8();
     }
   }
   // keys 8 lg .. 8 lg + 7 of channel dt * 16 + r: half lg / 2, chunk lg % 2, swapped for channels 8 .. 15
@@ -634,8 +600,8 @@ __device__ __forceinline__ void attend_block(BlockShared<GROUPS>& sh, int item, 
       a = max(a, __shfl_xor(a, o, QVL_WAVE));
       b = min(b, __shfl_xor(b, o, QVL_WAVE));
     }
-    w.all_lo = a;
-    w.all_hi = b;
+    w.all_lo = __builtin_amdgcn_readfirstlane(a);   // the same in every lane: compared in scalar registers
+    w.all_hi = __builtin_amdgcn_readfirstlane(b);
   }
   BlockLoader<GROUPS> ld;
   ld.bt = bt + (size_t)r * table_width;
@@ -660,26 +626,41 @@ __device__ __forceinline__ void attend_block(BlockShared<GROUPS>& sh, int item, 
       ++issued;
       if (issued < nblk) ld.next_pages(pg);
     }
-  for (int i = 0; i < rounds; ++i) {
-    // block i has landed when only the loads of the blocks issued after it are outstanding
-    const int later = issued - 1 - i;
-    if (later >= 2) wait_loads<2 * WAVE_LOADS>();
-    else if (later == 1) wait_loads<WAVE_LOADS>();
-    else wait_loads<0>();
+  // the rounds in which this wave's columns see keys of the block: i_first .. i_last (block kb0 + GROUPS i
+  // holds keys 32 kb .. 32 kb + 31; a wave without tiles has lo > hi and takes part in none)
+  const int lo_s = __builtin_amdgcn_readfirstlane(lo), hi_s = __builtin_amdgcn_readfirstlane(hi);
+  const int i_first = lo_s > hi_s ? rounds : ((lo_s >> 5) - kb0 + GROUPS - 1 < 0 ? 0 : ((lo_s >> 5) - kb0 + GROUPS - 1) / GROUPS);
+  const int i_last = lo_s > hi_s || (hi_s >> 5) < kb0 ? -1 : ((hi_s >> 5) - kb0) / GROUPS;
+  // One round: wait for block i, issue the loads of the block BLK_STAGES - 1 ahead, compute block i.
+  // In a steady round that block exists, so two blocks are in flight behind block i and nothing has
+  // to be asked (the table entry looked up for the block after the walk's last is never used).
+  auto round = [&](int i, auto steady_round) {
+    constexpr bool steady = decltype(steady_round)::value;
+    if constexpr (steady) {
+      wait_loads<2 * WAVE_LOADS>();
+    } else {
+      // block i has landed when only the loads of the blocks issued after it are outstanding
+      const int later = issued - 1 - i;
+      if (later >= 2) wait_loads<2 * WAVE_LOADS>();
+      else if (later == 1) wait_loads<WAVE_LOADS>();
+      else wait_loads<0>();
+    }
     __syncthreads();   // everybody's part of block i is there, and everybody has left block i - 1
-    if (issued < nblk) {
+    if (steady || issued < nblk) {
       ld.issue(pg, lds0 + (uint32_t)(issued % BLK_STAGES) * (STAGE_ELEMS * 2));   // into the stage of block i - 1
       ++issued;
-      if (issued < nblk) ld.next_pages(pg);
+      if (steady || issued < nblk) ld.next_pages(pg);
     }
-    const int kb = kb0 + GROUPS * i;
-    if (i < nblk && (kb << 5) + 31 >= lo && (kb << 5) <= hi) {
+    if (i >= i_first && i <= i_last) {
       const bf16_t* stage = sh.stage[group][i % BLK_STAGES];
       BlockRegs ops;
       operands_from_lds(stage, stage + K_LOADS * 512, ops);
-      w.template compute<true>(kb, qb, ops, st);
+      w.template compute<true>(kb0 + GROUPS * i, qb, ops, st);
     }
-  }
+  };
+  int i = 0;
+  for (; i < nblk - (BLK_STAGES - 1); ++i) round(i, std::true_type{});
+  for (; i < rounds; ++i) round(i, std::false_type{});
   if (GROUPS > 1) {
     // The second group's sums reach the first through the second group's stages, which nobody reads
     // or fills any more: word (tile, register, wave, lane), so every lane finds its partner's.
