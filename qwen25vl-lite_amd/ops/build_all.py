@@ -25,6 +25,10 @@ LIBRARIES = [
     ("attention_mfma", {"HD": 48}),
     ("attention_mfma", {"HD": 80}),
     ("attention_mfma", {"HD": 256}),
+    ("attention_mfma", {"HD": 32}),
+    ("attention_mfma", {"HD": 64}),
+    ("attention_mfma", {"HD": 96}),
+    ("attention_mfma", {"HD": 112}),
 ]
 
 

@@ -215,11 +215,13 @@ def test_paged_attention_matrix_cores(nq, nkv, hd, window, ps, split, monkeypatc
 
 @pytest.mark.parametrize("nq, nkv, hd, window, ps", [(28, 4, 128, None, 16), (6, 2, 48, 100, 16), (4, 4, 256, 257, 16),
                                                      (5, 1, 16, None, 16), (28, 4, 128, None, 48), (6, 2, 48, 100, 32),
-                                                     (4, 4, 256, 257, 64)])
+                                                     (4, 4, 256, 257, 64), (4, 2, 32, None, 16), (8, 2, 64, 70, 32),
+                                                     (3, 1, 96, None, 16), (6, 3, 112, 200, 48)])
 def test_paged_attention_long_portions(nq, nkv, hd, window, ps):
     """Prompt portions long enough for several blocks of several waves per request, next to a
     short portion and a decoded token: the kernel that shares keys through LDS walks the union of
-    its waves' ranges, with blocks that some of its waves skip."""
+    its waves' ranges, with blocks that some of its waves skip.  Every head size in steps of 16 up to
+    128 lays its stages out differently (loads per part, the second half's offset): all of them run."""
     from qwen25vl_lite_amd.ops import attention_mfma, kernels
     from qwen25vl_lite_amd.parts import StepContext
     lens, qlens = (413, 150, 90), (380, 3, 1)
