@@ -22,6 +22,7 @@ _MAX_HD = 256
 TARGET_BLOCKS = 512        # from here on a wave per tile fills the 256 compute units
 FILL_BLOCKS = 256          # with fewer cooperative blocks than this, long contexts are split
 MIN_KEYS_PER_SPLIT = 1024  # a split is worth a second kernel only above this many keys
+ALONE_KEYS = 4096          # decoded tokens beside prompt portions get a launch of their own from this context on
 
 
 def supports(head_dim: int, dtype: torch.dtype) -> bool:
@@ -81,14 +82,36 @@ def _work_queue(device: torch.device):
     return _queues[key]
 
 
-def _step_tiles(step, group: int, tile_ct: int, device, by_length: bool = False):
+def _step_tiles(step, group: int, tile_ct: int, device, by_length: bool = False, only=None):
+    """The step's entries on the device; ``only``: a tuple of 0/1 per request, entries of the others left out."""
     cache = step.derived
-    key = ("tiles", group, tile_ct, by_length)
+    key = ("tiles", group, tile_ct, by_length, only)
     if key not in cache:
         req, ct = tiles_for(step.cu_q_host, group, tile_ct, step.ctx_len_host if by_length else None)
+        if only is not None:
+            keep = np.asarray(only, dtype=bool)[req]
+            req, ct = req[keep], ct[keep]
         both = torch.from_numpy(np.concatenate([req, ct])).to(device, non_blocking=True)
         cache[key] = (both[:len(req)], both[len(req):], len(req))
     return cache[key]
+
+
+def long_single_tiles(step, group: int, nkv: int):
+    """In a step that has prompt portions too: the requests whose tokens make one tile only
+    (decoded tokens) if they are few and their contexts long, as a tuple of 0/1 per request, else
+    None.  Planned together with the portions, each of them gets one workgroup (or one block) that
+    walks its whole context, and that walk is what the step then waits for; in a launch of their
+    own their contexts are split among blocks (measured at the 7B decoder's heads: 8 decoded tokens
+    at 8,192 keys beside a portion of 256 take 87 us together, 32 and 13 apart).  Below
+    ``ALONE_KEYS`` the two launches, one after the other, cost more than the walks they shorten."""
+    q = np.diff(np.asarray(step.cu_q_host, dtype=np.int64))
+    single = (q > 0) & (q * group <= 16)
+    if not single.any() or single.all():
+        return None
+    longest = int(np.asarray(step.ctx_len_host, dtype=np.int64)[single].max())
+    if longest < ALONE_KEYS or int(single.sum()) * nkv >= FILL_BLOCKS:
+        return None
+    return tuple(int(x) for x in single)
 
 
 def block_groups(walks: int, places: int, head_dim: int) -> int:
@@ -119,20 +142,22 @@ def try_attention(q, k_cache, v_cache, block_table, step, num_q_heads: int, wind
     out = torch.empty_like(q)
     defines = {"HD": hd}
     kind, nsplit, per = plan_splits(num_tiles, nkv, step.max_ctx_len)
-    if kind == "tile":
-        tile_req, tile_ct, num_tiles = _step_tiles(step, nq // nkv, block_tiles(hd), q.device, by_length=True)
-    common = [_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(step.cu_q),
-              _ptr(step.ctx_len), _ptr(tile_req), _ptr(tile_ct), num_tiles, _ptr(out)]
-    if kind == "tile":
+
+    def many_tiles(only):
+        tile_req, tile_ct, num_tiles = _step_tiles(step, nq // nkv, block_tiles(hd), q.device, by_length=True, only=only)
         fn = _fn("attention_mfma", "qvl_attn_mfma_block",
                  [_c_ptr] * 4 + [_c_int] + [_c_ptr] * 4 + [_c_int, _c_ptr] + [_c_int] * 4
                  + [_c_float, _c_ptr, _c_int, _c_int, _c_ptr], defines)
         queue, cus = _work_queue(q.device)
         per_cu = int(_fn("attention_mfma", "qvl_attn_mfma_block_per_cu", [], defines)())
         groups = block_groups(num_tiles * nkv, cus * per_cu, hd) if force_groups is None else force_groups
-        _check(fn(*common, nq, nkv, ps, int(window or 0), float(scale), _ptr(queue),
-                  cus * (per_cu if groups == 1 else 1), groups, _stream()), "paged_attention (matrix cores)")
-    else:
+        _check(fn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(step.cu_q),
+                  _ptr(step.ctx_len), _ptr(tile_req), _ptr(tile_ct), num_tiles, _ptr(out), nq, nkv, ps, int(window or 0),
+                  float(scale), _ptr(queue), cus * (per_cu if groups == 1 else 1), groups, _stream()),
+               "paged_attention (matrix cores)")
+
+    def shared_tiles(only, nsplit, per):
+        tile_req, tile_ct, num_tiles = _step_tiles(step, nq // nkv, 1, q.device, only=only)
         scratch = None
         if nsplit > 1:
             floats = _fn("attention_mfma", "qvl_attn_mfma_scratch_floats", [_c_int] * 3, defines)
@@ -141,6 +166,25 @@ def try_attention(q, k_cache, v_cache, block_table, step, num_q_heads: int, wind
         fn = _fn("attention_mfma", "qvl_attn_mfma_coop",
                  [_c_ptr] * 4 + [_c_int] + [_c_ptr] * 4 + [_c_int, _c_ptr, _c_ptr] + [_c_int] * 4
                  + [_c_float, _c_int, _c_int, _c_ptr], defines)
-        _check(fn(*common, _ptr(scratch), nq, nkv, ps, int(window or 0), float(scale), nsplit, per, _stream()),
+        _check(fn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(step.cu_q),
+                  _ptr(step.ctx_len), _ptr(tile_req), _ptr(tile_ct), num_tiles, _ptr(out), _ptr(scratch), nq, nkv, ps,
+                  int(window or 0), float(scale), nsplit, per, _stream()),
                "paged_attention (matrix cores, shared tiles)")
+
+    single = long_single_tiles(step, nq // nkv, nkv) if force_groups is None else None
+    if single is not None:   # the few decoded tokens with long contexts by themselves, the rest planned anew
+        longest = max(c for c, s in zip(step.ctx_len_host, single) if s)
+        _, nsplit1, per1 = plan_splits(sum(single), nkv, longest)   # fewer blocks than FILL_BLOCKS: the kernel that splits
+        shared_tiles(single, nsplit1, per1)
+        rest = tuple(1 - s for s in single)
+        kind, nsplit, per = plan_splits(_step_tiles(step, nq // nkv, 1, q.device, only=rest)[2], nkv,
+                                        max(c for c, s in zip(step.ctx_len_host, rest) if s))
+        if kind == "tile":
+            many_tiles(rest)
+        else:
+            shared_tiles(rest, nsplit, per)
+    elif kind == "tile":
+        many_tiles(None)
+    else:
+        shared_tiles(None, nsplit, per)
     return out

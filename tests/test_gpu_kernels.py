@@ -213,6 +213,38 @@ def test_paged_attention_matrix_cores(nq, nkv, hd, window, ps, split, monkeypatc
     assert torch.allclose(out.float().cpu(), c["want"], atol=1.5e-2, rtol=2e-2), err
 
 
+@pytest.mark.parametrize("nq, nkv, hd, window", [(14, 2, 128, None), (6, 2, 48, 100)])
+def test_mixed_step_with_few_long_decoded_tokens(nq, nkv, hd, window, monkeypatch):
+    """A prompt portion beside two decoded tokens whose contexts are long: the decoded tokens go to
+    the kernel that splits a context among blocks, in a launch of their own, the portion to the
+    kernel for many tiles; both write into the same output.  (The limits are set low here so that
+    contexts of a few hundred keys count as long.)"""
+    from qwen25vl_lite_amd.ops import attention_mfma, kernels
+    from qwen25vl_lite_amd.parts import StepContext
+    lens, qlens = (333, 300, 17, 280), (40, 1, 17, 1)
+    c = _attention_case(torch.bfloat16, nq, nkv, hd, window, lens, qlens)
+    monkeypatch.setattr(attention_mfma, "TARGET_BLOCKS", 1)
+    monkeypatch.setattr(attention_mfma, "MIN_KEYS_PER_SPLIT", 64)
+    monkeypatch.setattr(attention_mfma, "ALONE_KEYS", 128)
+    cu = [0]
+    for ql in qlens:
+        cu.append(cu[-1] + ql)
+    none = torch.zeros(0, dtype=torch.int32).cuda()
+    step = StepContext(num_tokens=cu[-1], num_reqs=len(lens), token_ids=none, positions=none, token_req=c["req"],
+                       token_seqpos=c["seqpos"], cu_q=torch.tensor(cu, dtype=torch.int32).cuda(),
+                       ctx_len=torch.tensor(lens, dtype=torch.int32).cuda(), req_slots=none, groups=[],
+                       logit_rows=none, cu_q_host=cu, ctx_len_host=list(lens), max_q_len=max(qlens),
+                       max_ctx_len=max(lens), dtype=torch.bfloat16)
+    assert attention_mfma.long_single_tiles(step, nq // nkv, nkv) == (0, 1, 0, 1)
+    called = []
+    real = attention_mfma._fn
+    monkeypatch.setattr(attention_mfma, "_fn", lambda stem, name, *a, **k: (called.append(name), real(stem, name, *a, **k))[1])
+    out = attention_mfma.try_attention(c["q"], c["kc"], c["vc"], c["table"], step, nq, window, c["scale"])
+    assert "qvl_attn_mfma_coop" in called and "qvl_attn_mfma_block" in called
+    err = (out.float().cpu() - c["want"]).abs().max()
+    assert torch.allclose(out.float().cpu(), c["want"], atol=1.5e-2, rtol=2e-2), err
+
+
 @pytest.mark.parametrize("nq, nkv, hd, window, ps", [(28, 4, 128, None, 16), (6, 2, 48, 100, 16), (4, 4, 256, 257, 16),
                                                      (5, 1, 16, None, 16), (28, 4, 128, None, 48), (6, 2, 48, 100, 32),
                                                      (4, 4, 256, 257, 64), (4, 2, 32, None, 16), (8, 2, 64, 70, 32),
