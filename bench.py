@@ -71,6 +71,42 @@ def prefill_flops(t, tokens):
     return linear + attention + head
 
 
+def measure_attention(torch, size, lengths, page=16, reps=10):
+    """The causal attention of one prompt of each length, through the kernel that prompt portions take
+    (qwen25vl-lite_amd/csrc/attention_mfma.hip): mean time of ``reps`` calls and the rate of its
+    4 * heads * head_dim * T (T + 1) / 2 flops."""
+    from qwen25vl_lite_amd.ops import attention_mfma
+    from qwen25vl_lite_amd.parts import StepContext
+
+    nq, nkv = size["num_attention_heads"], size["num_key_value_heads"]
+    hd = size["hidden_size"] // nq
+    out = {"heads": nq, "kv_heads": nkv, "head_dim": hd, "page_size": page}
+    for T in lengths:
+        pages = (T + page - 1) // page
+        torch.manual_seed(0)
+        q = torch.randn(T, nq * hd, device="cuda").bfloat16()
+        kc = torch.randn(pages, nkv, page, hd, device="cuda").bfloat16()
+        vc = torch.randn(pages, nkv, hd, page, device="cuda").bfloat16()
+        table = torch.randperm(pages, device="cuda").int().view(1, pages)
+        none = torch.zeros(0, dtype=torch.int32, device="cuda")
+        ar = torch.arange(T, dtype=torch.int32, device="cuda")
+        step = StepContext(num_tokens=T, num_reqs=1, token_ids=none, positions=none, token_req=torch.zeros_like(ar),
+                           token_seqpos=ar, cu_q=torch.tensor([0, T], dtype=torch.int32, device="cuda"),
+                           ctx_len=torch.tensor([T], dtype=torch.int32, device="cuda"), req_slots=none, groups=[],
+                           logit_rows=none, cu_q_host=[0, T], ctx_len_host=[T], max_q_len=T, max_ctx_len=T,
+                           dtype=torch.bfloat16)
+        for _ in range(3):
+            attention_mfma.try_attention(q, kc, vc, table, step, nq, None, hd ** -0.5)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            attention_mfma.try_attention(q, kc, vc, table, step, nq, None, hd ** -0.5)
+        torch.cuda.synchronize()
+        sec = (time.perf_counter() - t0) / reps
+        out[f"tokens_{T}"] = {"us": round(sec * 1e6, 1), "tflops": round(4.0 * nq * hd * T * (T + 1) / 2 / sec / 1e12, 1)}
+    return out
+
+
 def measure_peaks(torch):
     """Plain read and copy rates, the matrix instruction's rate on registers and the cost of an empty
     launch, each the best of several repeats (kernels in qwen25vl-lite_amd/csrc/peaks.hip)."""
@@ -145,6 +181,9 @@ def main(argv=None) -> int:
     ap.add_argument("--peaks", action="store_true",
                     help="instead: what the device does at best (plain reads and copies, matrix instructions on "
                          "registers, an empty launch), for the fractions above to be read against")
+    ap.add_argument("--attention", type=int, nargs="+", metavar="TOKENS",
+                    help="instead: the prefill attention alone (one request of that many tokens in one step, the "
+                         "chosen size's heads, bfloat16, pages in shuffled order), microseconds and TFLOP/s for each length")
     ap.add_argument("--no-graph", action="store_true", help="do not replay decode steps from a HIP graph")
     ap.add_argument("--no-lookahead", action="store_true",
                     help="do not queue the next decode step before the running one's tokens are known")
@@ -158,6 +197,10 @@ def main(argv=None) -> int:
 
     if args.peaks:
         print(json.dumps(measure_peaks(torch)))
+        return 0
+
+    if args.attention:
+        print(json.dumps(measure_attention(torch, SIZES[args.size], args.attention)))
         return 0
 
     from qwen25vl_lite_amd import EngineConfig, LLMEngine, ModelRunner, Qwen25VLConfig, SamplingParams, build_model
