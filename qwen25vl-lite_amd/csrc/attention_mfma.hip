@@ -40,6 +40,18 @@ typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 #define KS ((HD + 31) / 32)  // 32-wide steps over the head for Q.K
 #define NT (HD / 16)         // 16-wide tiles of the head for P.V
+// The layout of a stage of the kernel for many tiles in LDS (described where that kernel begins).
+#define CH_PER_KEY (HD / 8)                                       // 16-byte chunks of a key
+#define KROW (HD + 8)                                             // elements of a K row in LDS
+#define K_SKEW ((4 * (CH_PER_KEY + 1)) % 16)                      // 16-byte slots by which the second half's rows are set off
+#define KH_LOADS ((16 * (CH_PER_KEY + 1) + K_SKEW + 63) / 64)     // 1 KB wave loads that cover the K rows of one half
+#define K_LOADS (2 * KH_LOADS)
+#define V_HALF_SLOTS ((2 * HD + 63) / 64 * 64)                    // slots of one half of the V^T rows (whole loads)
+#define VH_LOADS (V_HALF_SLOTS / 64)
+#define V_LOADS (2 * VH_LOADS)
+#define STAGE_LOADS (K_LOADS + V_LOADS)
+#define WAVE_LOADS (KH_LOADS > VH_LOADS ? KH_LOADS : VH_LOADS)    // what a wave issues a block: one of the four parts of a stage
+#define STAGE_ELEMS (STAGE_LOADS * 512)
 #define LOG2E 1.4426950408889634f
 
 __device__ __forceinline__ bf16x8_t load8(const bf16_t* p) {
@@ -255,6 +267,76 @@ struct Walk {
       }
     }
   }
+
+  // The same arithmetic for a wave that carries more column tiles than its registers hold operands
+  // for: the K rows and V^T rows of the stage (ks, vs) pass through a few registers, each fragment
+  // multiplied with every tile before the next is read; scores of all tiles, then the probabilities
+  // of all tiles, then the sums.  The way of the kernel for many tiles (see compute<true>).
+  __device__ __forceinline__ void compute_streamed(int kb, const bf16x8_t (*qb)[KS], const bf16_t* ks, const bf16_t* vs,
+                                                   TileState* sts) const {
+    const int key0 = kb << 5;
+    const bool interior = key0 >= all_lo && key0 + 31 <= all_hi;
+    f32x4_t s[CT][2];
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const bf16_t* row = ks + (r >> 3) * (KH_LOADS * 512 + K_SKEW * 8) + (8 * ((r >> 2) & 1) + 4 * b + (r & 3)) * KROW;
+#pragma unroll
+      for (int t = 0; t < CT; ++t) s[t][b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int q = 0; q < KS; ++q) {
+        const int d = q * 32 + 8 * lg;
+        const bf16x8_t k = (d < HD) ? load8(row + d) : zero8();
+#pragma unroll
+        for (int t = 0; t < CT; ++t) s[t][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k, qb[t][q], s[t][b], 0, 0, 0);
+      }
+    }
+    bf16x8_t pb[CT];
+#pragma unroll
+    for (int t = 0; t < CT; ++t) {
+      TileState& st = sts[t];
+      float raw[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) raw[j] = (j < 4) ? s[t][0][j] : s[t][1][j - 4];
+      if (!interior) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int key = key0 + 8 * lg + j;
+          const bool ok = key >= my_lo[t] && key <= my_p[t] && key >= key_begin && key <= key_end;
+          raw[j] = ok ? raw[j] : -INFINITY;
+        }
+      }
+      float mloc = max2(max2(max2(raw[0], raw[1]), max2(raw[2], raw[3])),
+                        max2(max2(raw[4], raw[5]), max2(raw[6], raw[7]))) * scale_log2;
+      if (__any(mloc > st.m + LAZY_LOG2)) {
+        mloc = max_over_groups(mloc);
+        const bool move = mloc > st.m + LAZY_LOG2;
+        const float m_new = move ? mloc : st.m;
+        const float alpha = move ? __builtin_amdgcn_exp2f(st.m - m_new) : 1.f;
+        st.m = m_new;
+#pragma unroll
+        for (int dt = 0; dt <= NT; ++dt) {
+          f32x4_t o = st.acc[dt];
+          o[0] *= alpha; o[1] *= alpha; o[2] *= alpha; o[3] *= alpha;
+          st.acc[dt] = o;
+        }
+      }
+      float nref = -st.m;
+      if (!interior) nref = st.m == -INFINITY ? 0.f : nref;
+      float pv[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) pv[j] = __builtin_amdgcn_exp2f(fmaf(raw[j], scale_log2, nref));
+      u32x4_t packed = {pack2(pv[0], pv[1]), pack2(pv[2], pv[3]), pack2(pv[4], pv[5]), pack2(pv[6], pv[7])};
+      pb[t] = __builtin_bit_cast(bf16x8_t, packed);
+      st.acc[NT] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones8(), pb[t], st.acc[NT], 0, 0, 0);
+    }
+    const int vslot = (lg >> 1) * V_HALF_SLOTS + 2 * r + ((lg & 1) ^ (r >> 3));
+#pragma unroll
+    for (int dt = 0; dt < NT; ++dt) {
+      const bf16x8_t v = load8(vs + (vslot + 32 * dt) * 8);
+#pragma unroll
+      for (int t = 0; t < CT; ++t) sts[t].acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, pb[t], sts[t].acc[dt], 0, 0, 0);
+    }
+  }
 };
 
 // Walk the 32-key blocks first, first + stride, ... that overlap keys [key_begin, key_end]
@@ -393,24 +475,19 @@ __device__ __forceinline__ void init_state(TileState& st) {
 // plain kind's independent workgroups overlap their matrix and vector phases better.
 #define BLK_WAVES 4
 #if HD <= 128
+#ifndef BLK_CT
 #define BLK_CT 2
+#endif
+#if BLK_CT > 2
+#define BLK_MAX_GROUPS 1
+#else
 #define BLK_MAX_GROUPS 2
+#endif
 #else
 #define BLK_CT 1
 #define BLK_MAX_GROUPS 1
 #endif
 #define BLK_STAGES 4
-#define CH_PER_KEY (HD / 8)                                       // 16-byte chunks of a key
-#define KROW (HD + 8)                                             // elements of a K row in LDS
-#define K_SKEW ((4 * (CH_PER_KEY + 1)) % 16)                      // 16-byte slots by which the second half's rows are set off
-#define KH_LOADS ((16 * (CH_PER_KEY + 1) + K_SKEW + 63) / 64)     // 1 KB wave loads that cover the K rows of one half
-#define K_LOADS (2 * KH_LOADS)
-#define V_HALF_SLOTS ((2 * HD + 63) / 64 * 64)                    // slots of one half of the V^T rows (whole loads)
-#define VH_LOADS (V_HALF_SLOTS / 64)
-#define V_LOADS (2 * VH_LOADS)
-#define STAGE_LOADS (K_LOADS + V_LOADS)
-#define WAVE_LOADS (KH_LOADS > VH_LOADS ? KH_LOADS : VH_LOADS)    // what a wave issues a block: one of the four parts of a stage
-#define STAGE_ELEMS (STAGE_LOADS * 512)
 #if 2 * WAVE_LOADS > 63
 #error "the in-flight loads of a wave do not fit the vmcnt counter"
 #endif
@@ -653,9 +730,13 @@ __device__ __forceinline__ void attend_block(BlockShared<GROUPS>& sh, int item, 
     }
     if (i >= i_first && i <= i_last) {
       const bf16_t* stage = sh.stage[group][i % BLK_STAGES];
-      BlockRegs ops;
-      operands_from_lds(stage, stage + K_LOADS * 512, ops);
-      w.template compute<true>(kb0 + GROUPS * i, qb, ops, st);
+      if constexpr (BLK_CT >= 3) {
+        w.compute_streamed(kb0 + GROUPS * i, qb, stage, stage + K_LOADS * 512, st);
+      } else {
+        BlockRegs ops;
+        operands_from_lds(stage, stage + K_LOADS * 512, ops);
+        w.template compute<true>(kb0 + GROUPS * i, qb, ops, st);
+      }
     }
   };
   int i = 0;

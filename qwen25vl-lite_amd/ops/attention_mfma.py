@@ -23,6 +23,9 @@ TARGET_BLOCKS = 512        # from here on a wave per tile fills the 256 compute 
 FILL_BLOCKS = 256          # with fewer cooperative blocks than this, long contexts are split
 MIN_KEYS_PER_SPLIT = 1024  # a split is worth a second kernel only above this many keys
 ALONE_KEYS = 4096          # decoded tokens beside prompt portions get a launch of their own from this context on
+WIDE_WALKS = 768           # the kind of the kernel whose waves carry three column tiles: from this many walks on
+WIDE_BLOCKS = 150_000      # ... that have this many 32-key blocks to walk between them
+WIDE_CT = 3
 
 
 def supports(head_dim: int, dtype: torch.dtype) -> bool:
@@ -31,9 +34,18 @@ def supports(head_dim: int, dtype: torch.dtype) -> bool:
 
 
 
-def block_tiles(head_dim: int) -> int:
+def block_tiles(head_dim: int, wide: bool = False) -> int:
     """Column tiles of one entry of the block list (BLK_WAVES * BLK_CT in the source)."""
-    return int(_fn("attention_mfma", "qvl_attn_mfma_block_tiles", [], {"HD": head_dim})())
+    return int(_fn("attention_mfma", "qvl_attn_mfma_block_tiles", [], block_defines(head_dim, wide))())
+
+
+def block_defines(head_dim: int, wide: bool) -> dict:
+    """The library of the kernel for many tiles: compiled per head size, and for head sizes up to 128
+    in a second kind whose waves carry three column tiles instead of two.  That kind reads its operands
+    from LDS once for three tiles (a third less LDS traffic and bookkeeping per product) at the price
+    of longer walks and no second group of waves: 6 % faster from about 8,192 prompt tokens on at the
+    7B decoder's heads, slower below."""
+    return {"HD": head_dim, "BLK_CT": WIDE_CT} if wide and head_dim <= 128 else {"HD": head_dim}
 
 
 def tiles_for(cu_q, group: int, tile_ct: int = 1, ctx_len=None) -> Tuple[np.ndarray, np.ndarray]:
@@ -96,6 +108,16 @@ def _step_tiles(step, group: int, tile_ct: int, device, by_length: bool = False,
     return cache[key]
 
 
+def _walk_blocks(step, group: int, tile_ct: int, only=None) -> int:
+    """About how many 32-key blocks the step's entries of ``tile_ct`` column tiles walk, for one key/value head."""
+    q = np.diff(np.asarray(step.cu_q_host, dtype=np.int64))
+    ctx = np.asarray(step.ctx_len_host, dtype=np.int64)
+    if only is not None:
+        q = q * np.asarray(only, dtype=np.int64)
+    entries = (q * group + 16 * tile_ct - 1) // (16 * tile_ct)
+    return int((entries * np.maximum(1, (ctx - q // 2 + 31) // 32)).sum())
+
+
 def long_single_tiles(step, group: int, nkv: int):
     """In a step that has prompt portions too: the requests whose tokens make one tile only
     (decoded tokens) if they are few and their contexts long, as a tuple of 0/1 per request, else
@@ -124,10 +146,10 @@ def block_groups(walks: int, places: int, head_dim: int) -> int:
 
 
 def try_attention(q, k_cache, v_cache, block_table, step, num_q_heads: int, window: Optional[int],
-                  scale: float, force_groups: Optional[int] = None) -> Optional[torch.Tensor]:
+                  scale: float, force_groups: Optional[int] = None, force_wide: Optional[bool] = None) -> Optional[torch.Tensor]:
     """The attention through the matrix-core kernel, or None if it does not take this shape.
-    ``force_groups`` (tests): the workgroup kind of the kernel for prompt portions, else chosen by
-    :func:`block_groups`."""
+    ``force_groups``, ``force_wide`` (tests): the workgroup kind of the kernel for prompt portions and
+    whether its waves carry three column tiles, else chosen by :func:`block_groups` and the number of walks."""
     pages, nkv, ps, hd = k_cache.shape
     if not supports(hd, q.dtype) or ps % 16:
         return None
@@ -145,12 +167,20 @@ def try_attention(q, k_cache, v_cache, block_table, step, num_q_heads: int, wind
 
     def many_tiles(only):
         tile_req, tile_ct, num_tiles = _step_tiles(step, nq // nkv, block_tiles(hd), q.device, by_length=True, only=only)
+        wide = force_wide
+        if wide is None:   # many and long walks: measured at the 7B decoder's heads, the wide kind wins from one prompt of about 8,192 tokens on
+            wide = hd <= 128 and num_tiles * nkv >= WIDE_WALKS and _walk_blocks(step, nq // nkv, block_tiles(hd), only) * nkv >= WIDE_BLOCKS
+        defines = block_defines(hd, wide)
+        if wide:
+            tile_req, tile_ct, num_tiles = _step_tiles(step, nq // nkv, block_tiles(hd, True), q.device, by_length=True, only=only)
         fn = _fn("attention_mfma", "qvl_attn_mfma_block",
                  [_c_ptr] * 4 + [_c_int] + [_c_ptr] * 4 + [_c_int, _c_ptr] + [_c_int] * 4
                  + [_c_float, _c_ptr, _c_int, _c_int, _c_ptr], defines)
         queue, cus = _work_queue(q.device)
         per_cu = int(_fn("attention_mfma", "qvl_attn_mfma_block_per_cu", [], defines)())
+        most = int(_fn("attention_mfma", "qvl_attn_mfma_block_max_groups", [], defines)())
         groups = block_groups(num_tiles * nkv, cus * per_cu, hd) if force_groups is None else force_groups
+        groups = min(groups, most) if force_groups is None else groups
         _check(fn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(step.cu_q),
                   _ptr(step.ctx_len), _ptr(tile_req), _ptr(tile_ct), num_tiles, _ptr(out), nq, nkv, ps, int(window or 0),
                   float(scale), _ptr(queue), cus * (per_cu if groups == 1 else 1), groups, _stream()),

@@ -29,6 +29,9 @@ LIBRARIES = [
     ("attention_mfma", {"HD": 64}),
     ("attention_mfma", {"HD": 96}),
     ("attention_mfma", {"HD": 112}),
+    # the kind whose waves carry three column tiles (long prompts)
+    ("attention_mfma", {"HD": 128, "BLK_CT": 3}),
+    ("attention_mfma", {"HD": 48, "BLK_CT": 3}),
 ]
 
 

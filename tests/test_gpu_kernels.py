@@ -271,9 +271,16 @@ def test_paged_attention_long_portions(nq, nkv, hd, window, ps):
     for groups in (1, 2) if hd <= 128 else (1,):   # an odd and an even number of key blocks among the walks
         with mock.patch.object(attention_mfma, "plan_splits", lambda t, n, m: ("tile", 1, 0)):
             out = attention_mfma.try_attention(c["q"], c["kc"], c["vc"], c["table"], step, nq, window, c["scale"],
-                                               force_groups=groups)
+                                               force_groups=groups, force_wide=False)
         err = (out.float().cpu() - c["want"]).abs().max()
         assert torch.allclose(out.float().cpu(), c["want"], atol=1.5e-2, rtol=2e-2), (groups, err)
+    if hd in (128, 48):   # the kind whose waves carry three column tiles (its operands pass through a few registers)
+        with mock.patch.object(attention_mfma, "plan_splits", lambda t, n, m: ("tile", 1, 0)):
+            out = attention_mfma.try_attention(c["q"], c["kc"], c["vc"], c["table"], step, nq, window, c["scale"],
+                                               force_groups=1, force_wide=True)
+        err = (out.float().cpu() - c["want"]).abs().max()
+        assert torch.allclose(out.float().cpu(), c["want"], atol=1.5e-2, rtol=2e-2), ("wide", err)
+        assert attention_mfma.block_tiles(hd, True) == 12 and attention_mfma.block_tiles(hd) == 8
     assert attention_mfma.block_groups(10, 512, hd) == (2 if hd <= 128 else 1)
     assert attention_mfma.block_groups(513, 512, hd) == 1
     with mock.patch.object(attention_mfma, "plan_splits", lambda t, n, m: ("tile", 1, 0)), pytest.raises(kernels.KernelError):
