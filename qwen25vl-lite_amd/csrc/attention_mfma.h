@@ -5,7 +5,9 @@
 #include <hip/hip_runtime.h>
 
 // Floats in the library's own array for partial results: 8 MiB, held on every GPU the library
-// runs on until the process ends.
+// runs on until the process ends.  The library is compiled once per head size (and once more for
+// its wide kind): every such variant that a process loads carries an array of its own, so a
+// process that uses n head sizes holds n times 8 MiB per GPU.
 #define QVL_ATTN_STATIC_SCRATCH_FLOATS (2 * 1024 * 1024)
 
 extern "C" {

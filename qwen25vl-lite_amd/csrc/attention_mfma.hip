@@ -25,6 +25,7 @@
 #include "common.h"
 #include <type_traits>
 #include "attention_mfma.h"
+#include <atomic>
 #include <mutex>
 
 #ifndef HD
@@ -494,7 +495,7 @@ __device__ __forceinline__ void init_state(TileState& st) {
 
 // The LDS address is stage + offset: added straight into M0.
 __device__ __forceinline__ void load16_to_lds(const char* base, uint32_t lane_bytes, uint32_t stage, uint32_t offset) {
-  asm volatile("s_add_i32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_bytes), "s"(base), "s"(stage), "s"(offset) : "memory", "scc");
+  asm volatile("s_add_i32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_bytes), "s"(base), "s"(stage), "s"(offset) : "memory", "scc", "m0");
 }
 // Wait until at most n of this wave's loads are outstanding (they finish in order).
 template <int N>
@@ -1042,27 +1043,30 @@ extern "C" int qvl_attn_mfma_coop(const void* q, const void* kc, const void* vc,
 static __device__ __align__(256) float scratch[QVL_ATTN_STATIC_SCRATCH_FLOATS];
 
 #define QVL_MAX_DEVICES 64
-static float* scratch_of_device[QVL_MAX_DEVICES];
+static std::atomic<float*> scratch_of_device[QVL_MAX_DEVICES];
 static std::mutex scratch_lock;
 
-// The current device's copy of the array, or nullptr (then *err says why).
+// The current device's copy of the array, or nullptr (then *err says why).  After a device's first
+// call this is one atomic load: the lock is taken only while an address is still unknown.
 static float* static_scratch(int* err) {
   int dev = -1;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= QVL_MAX_DEVICES) {
     *err = QVL_ERR_LIMIT;
     return nullptr;
   }
+  float* ptr = scratch_of_device[dev].load(std::memory_order_acquire);
+  if (ptr) return ptr;
   std::lock_guard<std::mutex> hold(scratch_lock);
-  if (!scratch_of_device[dev]) {
-    float* ptr = nullptr;
+  ptr = scratch_of_device[dev].load(std::memory_order_relaxed);
+  if (!ptr) {
     if (hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) {
       (void)hipGetLastError();
       *err = QVL_ERR_LAUNCH;
       return nullptr;
     }
-    scratch_of_device[dev] = ptr;
+    scratch_of_device[dev].store(ptr, std::memory_order_release);
   }
-  return scratch_of_device[dev];
+  return ptr;
 }
 
 extern "C" long long qvl_attn_mfma_static_scratch_floats() { return QVL_ATTN_STATIC_SCRATCH_FLOATS; }

@@ -165,11 +165,18 @@ class _Graph:
             self.step.token_ids[:len(entries)].copy_(device_tokens)
         if self.graph is None:
             # twice eagerly (libraries pick kernels and workspaces, per-step tile lists are made),
-            # then once more under capture; a decode step only writes the step's own cache slots
-            # and the logits, so running it again with the same inputs changes nothing
+            # then once more under capture.  Keys and values go to the step's own cache slots and
+            # the logits to their buffer, so running the step again with the same inputs changes
+            # nothing there.  Per-request state of a mixer is another matter: every pass advances
+            # it.  The rows are copied aside first and put back after each eager pass, so that the
+            # replay below is the only pass that counts.
+            kept = [None if s is None else s.clone() for s in parts.states]
             for _ in range(2):
                 self.step.per_pass.clear()
                 parts.model.forward(self.step, parts.slots)
+                for s, k in zip(parts.states, kept):
+                    if s is not None:
+                        s.copy_(k)
             torch.cuda.synchronize()
             self.step.per_pass.clear()    # what a pass computes from the step's values is computed in the graph
             self.graph, self.logits = _capture(lambda: parts.model.forward(self.step, parts.slots))
@@ -203,6 +210,7 @@ class _RunnerParts:
         self.model = runner.model
         self.cache = runner.cache
         self.slots = runner.slots
+        self.states = runner.states
         self.device = runner.device
         self.dtype = runner.dtype
         self.pad_state_slot = runner.pad_state_slot

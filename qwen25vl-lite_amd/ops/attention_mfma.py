@@ -85,8 +85,10 @@ _queues = {}
 
 
 def _work_queue(device: torch.device):
-    """Per device: the counters of the block kernel's work queues (it leaves them at zero) and
-    how many workgroups fill the device."""
+    """Per device: the counters of the block kernel's work queues and how many workgroups fill
+    the device.  A launch finds the counters at zero and leaves them at zero; launches on one
+    device share them, so they must follow each other on one stream (the engine has one).  A launch
+    that reports an error has them cleared."""
     key = torch.device(device).index or 0
     if key not in _queues:
         cus = torch.cuda.get_device_properties(device).multi_processor_count
@@ -148,6 +150,8 @@ def block_groups(walks: int, places: int, head_dim: int) -> int:
 def try_attention(q, k_cache, v_cache, block_table, step, num_q_heads: int, window: Optional[int],
                   scale: float, force_groups: Optional[int] = None, force_wide: Optional[bool] = None) -> Optional[torch.Tensor]:
     """The attention through the matrix-core kernel, or None if it does not take this shape.
+    Calls on one device must not overlap (one stream): the kernel for prompt portions keeps its
+    work-queue counters in memory that all calls on the device share.
     ``force_groups``, ``force_wide`` (tests): the workgroup kind of the kernel for prompt portions and
     whether its waves carry three column tiles, else chosen by :func:`block_groups` and the number of walks."""
     pages, nkv, ps, hd = k_cache.shape
@@ -181,10 +185,13 @@ def try_attention(q, k_cache, v_cache, block_table, step, num_q_heads: int, wind
         most = int(_fn("attention_mfma", "qvl_attn_mfma_block_max_groups", [], defines)())
         groups = block_groups(num_tiles * nkv, cus * per_cu, hd) if force_groups is None else force_groups
         groups = min(groups, most) if force_groups is None else groups
-        _check(fn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(step.cu_q),
+        code = fn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(step.cu_q),
                   _ptr(step.ctx_len), _ptr(tile_req), _ptr(tile_ct), num_tiles, _ptr(out), nq, nkv, ps, int(window or 0),
-                  float(scale), _ptr(queue), cus * (per_cu if groups == 1 else 1), groups, _stream()),
-               "paged_attention (matrix cores)")
+                  float(scale), _ptr(queue), cus * (per_cu if groups == 1 else 1), groups, _stream())
+        if code:
+            # whatever a launch that went wrong did to the counters, the next one starts from zero
+            queue.zero_()
+        _check(code, "paged_attention (matrix cores)")
 
     def shared_tiles(only, nsplit, per):
         tile_req, tile_ct, num_tiles = _step_tiles(step, nq // nkv, 1, q.device, only=only)

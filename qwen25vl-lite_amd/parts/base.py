@@ -138,7 +138,11 @@ class ResidualStream:
 class Part:
     """Base of all parts.  ``graph_safe`` says that ``forward`` only launches device work whose
     shape depends on the step's shape alone (no host reads of device data, no host loops over
-    the step's values), so a decode step through it may be captured in a HIP graph."""
+    the step's values: requests, positions, state rows and pages are found through the step's
+    device tensors), so a decode step through it may be captured in a HIP graph and replayed
+    with other values in the same buffers.  It promises nothing about running a step twice: a
+    mixer may advance its per-request state on every pass (the engine puts the state rows back
+    after the passes it runs to warm a new graph up)."""
 
     graph_safe: bool = False
     takes_lazy_norm: bool = False   # forward accepts NormedRows in place of the normalised tensor

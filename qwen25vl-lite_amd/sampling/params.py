@@ -40,13 +40,14 @@ class SamplingParams:
     ignore_eos: bool = False
 
     def validate(self) -> None:
-        if self.temperature < 0:
-            raise ValueError("temperature must be >= 0")
-        if not 0.0 < self.top_p <= 1.0:
-            raise ValueError("top_p must be in (0, 1]")
-        if self.max_tokens <= 0:
-            raise ValueError("max_tokens must be positive")
-        if self.repetition_penalty <= 0:
-            raise ValueError("repetition_penalty must be positive")
-        if not 0.0 <= self.min_p <= 1.0:
-            raise ValueError("min_p must be in [0, 1]")
+        """Raise ValueError for a value outside its range, naming the field and the value."""
+        ranges = (
+            ("temperature", self.temperature >= 0, "zero (greedy) or more"),
+            ("top_p", 0.0 < self.top_p <= 1.0, "above 0 and at most 1"),
+            ("min_p", 0.0 <= self.min_p <= 1.0, "between 0 and 1"),
+            ("max_tokens", self.max_tokens >= 1, "at least one token"),
+            ("repetition_penalty", self.repetition_penalty > 0, "above 0 (1 switches it off)"),
+        )
+        for name, ok, wanted in ranges:
+            if not ok:
+                raise ValueError(f"SamplingParams.{name} = {getattr(self, name)!r}: expected {wanted}")

@@ -62,7 +62,19 @@ TINY_C = {
     "rope_scaling": {"type": "mrope", "mrope_section": [10, 6, 8]},
 }
 
-TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2)}
+# The 7B decoder's head geometry (28 query heads on 4 key/value heads of 128 channels, its rotation
+# sections) at a narrow width: the attention of a long context at the sizes the dispatch rules
+# were measured for, cheap enough for the plain implementation.
+TINY_D = {
+    "architectures": ["Qwen2_5_VLForConditionalGeneration"],
+    "tie_word_embeddings": True,
+    "hidden_size": 256, "intermediate_size": 520, "num_hidden_layers": 2, "num_attention_heads": 28,
+    "num_key_value_heads": 4, "head_dim": 128, "vocab_size": 300, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6,
+    "use_sliding_window": False, "sliding_window": 32768,
+    "rope_scaling": {"type": "mrope", "mrope_section": [16, 24, 24]},
+}
+
+TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (TINY_D, 3)}
 
 
 @pytest.fixture(scope="session")

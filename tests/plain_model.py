@@ -129,16 +129,21 @@ def plain_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: fl
     (reference attention.py:143-148).  q [heads, T, hd]; k, v [kv_heads, T, hd]."""
     heads, t, _ = q.shape
     groups = heads // k.shape[0]
-    kk = k.repeat_interleave(groups, dim=0)
-    vv = v.repeat_interleave(groups, dim=0)
-    scores = torch.matmul(q.float(), kk.float().transpose(-2, -1)) * scale
-    i = torch.arange(t)[:, None]
-    j = torch.arange(t)[None, :]
-    allowed = j <= i
-    if window is not None:
-        allowed = allowed & (i - j < window)
-    scores = scores.masked_fill(~allowed, float("-inf"))
-    return torch.matmul(torch.softmax(scores, dim=-1), vv.float())
+    kk = k.repeat_interleave(groups, dim=0).float()
+    vv = v.repeat_interleave(groups, dim=0).float()
+    out = []
+    rows = 1024   # queries are taken a slice at a time, only so that the score matrix of a long sequence fits memory
+    for lo in range(0, t, rows):
+        hi = min(t, lo + rows)
+        scores = torch.matmul(q[:, lo:hi].float(), kk[:, :hi].transpose(-2, -1)) * scale
+        i = torch.arange(lo, hi)[:, None]
+        j = torch.arange(hi)[None, :]
+        allowed = j <= i
+        if window is not None:
+            allowed = allowed & (i - j < window)
+        scores = scores.masked_fill(~allowed, float("-inf"))
+        out.append(torch.matmul(torch.softmax(scores, dim=-1), vv[:, :hi]))
+    return torch.cat(out, dim=1)
 
 
 def plain_mlp(x: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, down: torch.Tensor, store=_keep) -> torch.Tensor:

@@ -97,11 +97,12 @@ def mixed_trace(requests: Dict[str, List[int]], seed: int = 0, max_live: int = 4
     return steps, peak
 
 
-def run_steps(replayer, steps: List[dict], holders: Dict[Tuple[int, int], set] = None
-              ) -> Dict[Tuple[str, int], torch.Tensor]:
+def run_steps(replayer, steps: List[dict], holders: Dict[Tuple[int, int], set] = None,
+              at: Dict[str, int] = None) -> Dict[Tuple[str, int], torch.Tensor]:
     """Replay and return {(request, index in its sequence): logits row} on the host.  ``holders``,
-    if given, collects for every (cache group, page) the requests that held it at some time."""
-    at: Dict[str, int] = {}
+    if given, collects for every (cache group, page) the requests that held it at some time.
+    ``at`` (request -> tokens fed so far) lets a caller replay a trace in several calls."""
+    at = {} if at is None else at
     out: Dict[Tuple[str, int], torch.Tensor] = {}
     cache = replayer.runner.cache
     for rec in steps:

@@ -130,7 +130,9 @@ def _paged(k, v, ps, pages, dtype, seed):
     return kc, vc, table
 
 
-ATTN_SHAPES = [(6, 2, 24, None), (5, 1, 48, 40), (8, 8, 16, 7), (14, 2, 128, None), (4, 2, 80, 130)]
+# the last shape has more query heads to a key/value head (20) than a column tile has columns: a
+# token's heads span two tiles
+ATTN_SHAPES = [(6, 2, 24, None), (5, 1, 48, 40), (8, 8, 16, 7), (14, 2, 128, None), (4, 2, 80, 130), (40, 2, 64, None)]
 
 
 def _attention_case(dtype, nq, nkv, hd, window, lens=(333, 17, 64, 1), qlens=(5, 17, 1, 1), ps=16):
@@ -281,6 +283,9 @@ def test_paged_attention_long_portions(nq, nkv, hd, window, ps):
         err = (out.float().cpu() - c["want"]).abs().max()
         assert torch.allclose(out.float().cpu(), c["want"], atol=1.5e-2, rtol=2e-2), ("wide", err)
         assert attention_mfma.block_tiles(hd, True) == 12 and attention_mfma.block_tiles(hd) == 8
+    # every launch leaves the work-queue counters at zero for the next one
+    torch.cuda.synchronize()
+    assert int(attention_mfma._work_queue(c["q"].device)[0].abs().sum()) == 0
     assert attention_mfma.block_groups(10, 512, hd) == (2 if hd <= 128 else 1)
     assert attention_mfma.block_groups(513, 512, hd) == 1
     with mock.patch.object(attention_mfma, "plan_splits", lambda t, n, m: ("tile", 1, 0)), pytest.raises(kernels.KernelError):
@@ -536,6 +541,28 @@ def test_projection_with_rotation_and_cache_write_folded_in(m, nq, nkv, hd, k, b
         assert not torch.equal(kc_b, kc0) and not torch.equal(vc_b, vc0)
         touched = (kc_b != kc0).any(dim=3).any(dim=1).flatten().nonzero().flatten().tolist()
         assert set(touched) <= set(s for s in slots.tolist() if s >= 0)
+    # And against the plain formulas themselves (not another path of the engine): the frequencies'
+    # rows laid out by sections, the product in float32 on the host, the reference's rotation.
+    sections = (half - 2 * (half // 3), half // 3, half // 3)
+    rows = torch.tensor(sum(([r] * c for r, c in enumerate(sections)), []), dtype=torch.int32).cuda()
+    kc_c, vc_c = kc0.clone(), vc0.clone()
+    q_c = skinny.qkv_rope_product(w, kernels.rope_table(pos, inv_freq, rows, m), bias=b, slots=slots if nkv else None,
+                                  k_cache=kc_c if nkv else None, v_cache=vc_c if nkv else None, num_q_heads=nq,
+                                  num_kv_heads=nkv, head_dim=hd, page_size=ps, **src)
+    xb = x.float().cpu() @ w.float().cpu().T + (b.cpu() if bias else 0.0)
+    qs, ks, vs = xb.split([nq * hd, nkv * hd, nkv * hd], dim=1)
+    cos, sin = plain_mrope_cos_sin(pos.cpu(), inv_freq.cpu())
+    heads = lambda t, n: t.reshape(m, n, hd).transpose(0, 1)
+    qr, kr = plain_apply_mrope(heads(qs, nq), heads(ks, nkv) if nkv else heads(qs, nq), cos, sin, sections)
+    plain_tol = dict(atol=3e-2, rtol=2e-2)     # the norm's output and the result each rounded to bfloat16 once
+    assert torch.allclose(q_c.float().cpu().view(m, nq, hd), qr.transpose(0, 1), **plain_tol)
+    if nkv:
+        kflat = kc_c.float().cpu().permute(0, 2, 1, 3).reshape(pages * ps, nkv, hd)
+        vflat = vc_c.float().cpu().permute(0, 3, 1, 2).reshape(pages * ps, nkv, hd)
+        live = (slots >= 0).cpu()
+        at = slots.cpu().long()[live]
+        assert torch.allclose(kflat[at], kr.transpose(0, 1)[live], **plain_tol)
+        assert torch.allclose(vflat[at], vs.view(m, nkv, hd)[live], **plain_tol)
     # a head size whose rotation the kernel does not take, or a cache of another type, is refused
     assert not skinny.takes_qkv_rope(m, k, w, 24, 12, torch.bfloat16)
     assert not skinny.takes_qkv_rope(m, k, w, hd, half - 1, torch.bfloat16)

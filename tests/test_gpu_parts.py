@@ -212,14 +212,36 @@ def _register_toys():
         def __init__(self, params, dtype, device):
             super().__init__(dtype, device)
             self.theta = params["theta"]
+            self.tables = {}
 
         def rotary_tables(self, head_dim):
-            rot = head_dim // 2
-            inv = 0.5 * plain_inv_freq(rot, self.theta)
-            return inv.to(self.device), torch.full((rot // 2,), 2, dtype=torch.int32, device=self.device)
+            if head_dim not in self.tables:      # made once: a captured step must not copy from the host
+                rot = head_dim // 2
+                inv = 0.5 * plain_inv_freq(rot, self.theta)
+                self.tables[head_dim] = (inv.to(self.device),
+                                         torch.full((rot // 2,), 2, dtype=torch.int32, device=self.device))
+            return self.tables[head_dim]
+
+    class GraphDecayMixer(DecayMixer):
+        """The same mixer with a decode path that may be captured: the requests' state rows are
+        found through the step's device tensor, not through a host loop."""
+        graph_safe = True
+
+        def forward(self, x, step, slot):
+            if step.max_q_len != 1:
+                return super().forward(x, step, slot)
+            rows = step.req_slots.long()
+            s = self.a * slot.state.index_select(0, rows) + x.float() @ self.B.T
+            slot.state.index_copy_(0, rows, s)
+            return (s @ self.C.T).to(torch.float32)
+
+    class GraphRoutedFeedForward(RoutedFeedForward):
+        graph_safe = True
 
     register_part("mixer", "toy_decay", DecayMixer)
+    register_part("mixer", "toy_decay_graph", GraphDecayMixer)
     register_part("ffn", "toy_routed", RoutedFeedForward)
+    register_part("ffn", "toy_routed_graph", GraphRoutedFeedForward)
     register_part("position", "toy_half_speed", HalfSpeedRoPE)
 
 
@@ -332,21 +354,22 @@ TOY_CONFIG = {
 }
 
 
-def _register_toy_architecture():
+def _register_toy_architecture(name="ToyDecayLM", graph=""):
+    """``graph="_graph"``: the same architecture from the toy parts that may be captured."""
     from qwen25vl_lite_amd.config import known_architectures, register_architecture
     from qwen25vl_lite_amd.models import LayerSpec, ModelSpec, RunEntry
     from qwen25vl_lite_amd.parts import PartSpec
     _register_toys()
-    if "ToyDecayLM" in known_architectures():
+    if name in known_architectures():
         return
 
     def build_spec(cfg):
         hidden = cfg.width
         norm = PartSpec("rms_norm", {"size": hidden, "eps": 1e-6})
         pos = PartSpec("toy_half_speed", {"theta": cfg.base})
-        mixers = {"decay": PartSpec("toy_decay", {"hidden_size": hidden, "state_size": cfg.state}),
+        mixers = {"decay": PartSpec("toy_decay" + graph, {"hidden_size": hidden, "state_size": cfg.state}),
                   "attention": _attn_spec(hidden, cfg.heads, cfg.groups, cfg.head, pos, window=cfg.reach)}
-        ffns = {"routed": PartSpec("toy_routed", {"hidden_size": hidden}),
+        ffns = {"routed": PartSpec("toy_routed" + graph, {"hidden_size": hidden}),
                 "swiglu": PartSpec("swiglu", {"hidden_size": hidden, "intermediate_size": cfg.inner})}
         layers = []
         for i, (mixer, ffn) in enumerate(cfg.plan):
@@ -360,7 +383,7 @@ def _register_toy_architecture():
                          map_name=lambda name: name[4:] if name.startswith("toy.") else name,
                          eos_token_id=cfg.stop_id)
 
-    register_architecture("ToyDecayLM", build_spec)      # no reader of its own: the raw keys are its configuration
+    register_architecture(name, build_spec)      # no reader of its own: the raw keys are its configuration
 
 
 def test_toy_architecture_from_a_model_folder(tmp_path):
@@ -409,6 +432,38 @@ def test_toy_architecture_from_a_model_folder(tmp_path):
     for i, (a, b) in enumerate(((0, 9), (9, 11), (11, 23))):
         rows.append(rp.step({"step": i + 1, "entries": [{"id": "c", "tokens": toks[a:b], "want": list(range(b - a))}]}))
     assert torch.allclose(torch.cat(rows).cpu(), want, atol=2e-4)
+
+
+def test_a_stateful_mixer_under_decode_graphs(tmp_path):
+    """A mixer that keeps per-request state and says it may be captured: decode steps then run from
+    HIP graphs.  A new graph is warmed up by running its first step several times, each of which
+    advances the state; the engine must put the state rows back, or the tokens after the first
+    capture differ from the eager run's and the plain toy's.  Two batch sizes are captured (three
+    requests, then two once the shortest has ended)."""
+    from qwen25vl_lite_amd import LLM, SamplingParams, write_random_model
+    from qwen25vl_lite_amd.config import load_config
+    _register_toy_architecture("ToyDecayGraphLM", "_graph")
+    d = str(tmp_path / "toy_graph")
+    write_random_model(load_config(dict(TOY_CONFIG, architectures=["ToyDecayGraphLM"])), d, seed=11, std=0.3,
+                       dtype=torch.float32)
+    g = torch.Generator().manual_seed(6)
+    prompts = [torch.randint(0, 39, (n,), generator=g).tolist() for n in (5, 23, 12)]
+    params = [SamplingParams(temperature=0.0, max_tokens=n, ignore_eos=True) for n in (9, 4, 9)]
+    options = dict(dtype="float32", num_blocks=16, block_size=16, max_num_seqs=3, max_num_batched_tokens=64)
+    with LLM(d, hip_graph=True, **options) as llm:
+        assert llm.model.graph_safe and llm.runner.graphs is not None
+        outs = llm.generate(prompts, params)
+        assert len(llm.runner.graphs.graphs) >= 2, "decode steps of two batch sizes ran from graphs"
+        model = llm.model
+        for prompt, sp, out in zip(prompts, params, outs):
+            ids, want = list(prompt), []
+            for _ in range(sp.max_tokens):
+                nxt = int(torch.argmax(_plain_toy_model(model, ids, torch.arange(len(ids)))[-1]))
+                want.append(nxt)
+                ids.append(nxt)
+            assert out.output_token_ids == want
+    eager = LLM(d, hip_graph=False, **options)
+    assert [o.output_token_ids for o in eager.generate(prompts, params)] == [o.output_token_ids for o in outs]
 
 
 def test_a_block_with_two_mixers_gets_a_slot_for_each():

@@ -74,9 +74,12 @@ def test_replay_every_way(model_dirs, name, dtype, block_size):
         print(name, "bfloat16 against float32", _compare(got, _reference(d, requests), dtype, "whole/float32"))
     assert rp.runner.cache.pages_in_use() == [0] * len(rp.runner.cache.groups)
 
+    pure = _reference(d, requests) if dtype == "bfloat16" and "sharp" not in name else None
     got = run_steps(rp, tail_trace(requests))
     assert len(got) == total
     print(name, dtype, "tail", _compare(got, ref, dtype, "tail"))
+    if pure is not None:
+        print(name, "tail against float32", _compare(got, pure, dtype, "tail/float32"))
 
     got = run_steps(rp, portion_trace(requests))
     assert len(got) == total
@@ -89,6 +92,8 @@ def test_replay_every_way(model_dirs, name, dtype, block_size):
     got = run_steps(rp, steps, holders)
     assert len(got) == total
     print(name, dtype, "mixed", _compare(got, ref, dtype, "mixed"), "pool tokens", peak)
+    if pure is not None:
+        print(name, "mixed against float32", _compare(got, pure, dtype, "mixed/float32"))
     reused = sum(len(who) > 1 for who in holders.values())
     assert reused >= 2, "the trace must hand pages of finished requests to later ones"
     rp.runner.cache.check()

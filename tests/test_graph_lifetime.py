@@ -25,7 +25,7 @@ def _stub_runner():
     runner = types.SimpleNamespace(
         model=types.SimpleNamespace(spec=types.SimpleNamespace(position_rows=3)),
         cache=types.SimpleNamespace(groups=[], page_size=16), slots=[], device=torch.device("cpu"),
-        dtype=torch.float32, pad_state_slot=4,
+        dtype=torch.float32, pad_state_slot=4, states=[],
         ecfg=types.SimpleNamespace(max_blocks_per_seq=8, max_num_seqs=4))
     runner.graphs = DecodeGraphs(runner)
     return runner

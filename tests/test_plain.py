@@ -106,6 +106,16 @@ def test_attention_is_the_library_routine():
     # one head, no mask effect on the last row: plain softmax(q k^T) v
     last = torch.softmax((q[0, -1] @ k[0].T) * hd ** -0.5, -1) @ v[0]
     assert torch.allclose(got[0, -1], last, atol=1e-5)
+    # a sequence longer than the slice of queries the function takes at a time, with a window that
+    # reaches across slices
+    t = 1100
+    q, k, v = torch.randn(2, t, hd), torch.randn(1, t, hd), torch.randn(1, t, hd)
+    i, j = torch.arange(t)[:, None], torch.arange(t)[None, :]
+    for window in (None, 90):
+        mask = (j <= i) if window is None else (j <= i) & (i - j < window)
+        lib = F.scaled_dot_product_attention(q[None], k.repeat_interleave(2, 0)[None], v.repeat_interleave(2, 0)[None],
+                                             attn_mask=mask)[0]
+        assert torch.allclose(plain_attention(q, k, v, hd ** -0.5, window), lib, atol=1e-5)
 
 
 def test_window_edges():

@@ -116,3 +116,43 @@ def test_safetensors_roundtrip_against_the_library(tmp_path):
     with SafetensorsFile(str(tmp_path / "theirs.safetensors")) as f:
         for k, v in tensors.items():
             assert torch.equal(theirs[k], v) and torch.equal(f.tensor(k), v) and f.dtype(k) == v.dtype
+
+
+def test_a_folder_of_two_shards_with_an_index(tmp_path):
+    """Checkpoints of real size come as several files named by ``model.safetensors.index.json``
+    (reference model.py:312-348).  The same tensors in two shards (and a vision tensor that is
+    skipped) load to the very values of the single file; a tensor that no shard holds is
+    reported as missing."""
+    d = _folder(tmp_path, TINY_B, seed=5)
+    cfg = Qwen25VLConfig.from_pretrained(d)
+    single = build_model(cfg, torch.bfloat16, "cpu")
+    assert load_weights(d, single)["loaded"] == len(single.expected_tensors())
+    path = os.path.join(d, "model.safetensors")
+    with SafetensorsFile(path) as f:
+        tensors = {k: f.tensor(k).clone() for k in f.keys()}
+    names = sorted(tensors)
+    first, second = names[::2], names[1::2]
+    write_safetensors(os.path.join(d, "model-00001-of-00002.safetensors"), {k: tensors[k] for k in first})
+    write_safetensors(os.path.join(d, "model-00002-of-00002.safetensors"),
+                      {**{k: tensors[k] for k in second}, "visual.patch_embed.proj.weight": torch.zeros(3, 2)})
+    weight_map = {k: "model-00001-of-00002.safetensors" for k in first}
+    weight_map.update({k: "model-00002-of-00002.safetensors" for k in second})
+    with open(os.path.join(d, "model.safetensors.index.json"), "w") as fh:
+        json.dump({"metadata": {}, "weight_map": weight_map}, fh)
+    os.remove(path)
+    sharded = build_model(cfg, torch.bfloat16, "cpu")
+    counts = load_weights(d, sharded)
+    assert counts["loaded"] == len(sharded.expected_tensors()) and counts["skipped"] == 1
+    assert torch.equal(sharded.embed, single.embed) and torch.equal(sharded.head, single.head)
+    for a, b in zip(sharded.blocks, single.blocks):
+        for name, t in a.mixer.named_weights().items():
+            assert torch.equal(t, b.mixer.named_weights()[name]), name
+        for name, t in a.ffn.named_weights().items():
+            assert torch.equal(t, b.ffn.named_weights()[name]), name
+        assert torch.equal(a.norm1.weight, b.norm1.weight) and torch.equal(a.norm2.weight, b.norm2.weight)
+    # a shard that lost a tensor: one error that names it
+    lost = second[0]
+    write_safetensors(os.path.join(d, "model-00002-of-00002.safetensors"), {k: tensors[k] for k in second[1:]})
+    with pytest.raises(WeightsError) as err:
+        load_weights(d, build_model(cfg, torch.bfloat16, "cpu"))
+    assert err.value.missing == [map_checkpoint_name(lost)]
