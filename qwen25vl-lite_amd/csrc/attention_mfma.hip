@@ -844,7 +844,14 @@ __global__ __launch_bounds__(64 * BLK_WAVES * GROUPS, GROUPS == 1 ? BLK_PER_CU :
 // The COOP_WAVES waves of a block take the tile's 32-key blocks in turn (wave w the blocks
 // w, w + COOP_WAVES, ...), then merge their sums and statistics through LDS in wave order.  With
 // nsplit > 1 the key range is further cut among blocks (grid.z); each block then writes its
-// merged partial to scratch and a second kernel merges the splits.
+// merged partial to scratch.  The splits are merged by the block that finishes last (one counter
+// per (tile, kv head) tells a block whether it is that one), or, for callers without counters, by
+// a second kernel.
+// Blocks of one tile may run on different XCDs, whose L2 caches do not see each other's lines: the
+// partial results are stored and loaded at device scope (they go through to memory), every thread
+// waits for its stores before the block's barrier, and only then is the counter raised, by a
+// relaxed device-scope atomic.  No fence is used (a device-scope fence writes a whole L2 back).
+// The last block leaves the counter at zero for the next launch.
 // scratch layout per (tile, kv head, split): 16 columns x PART_COLS floats (HD sums, m, l, and
 // padding that keeps every column 16-byte aligned).
 #define PART_COLS (HD + 4)
@@ -855,12 +862,74 @@ __global__ __launch_bounds__(64 * BLK_WAVES * GROUPS, GROUPS == 1 ? BLK_PER_CU :
 #define COOP_WAVES 2
 #endif
 
+// Device-scope ("agent") stores and loads: visible across the XCDs' L2 caches.
+__device__ __forceinline__ void store_device_scope(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_device_scope(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Merge the nsplit partial results of one (tile, kv head) and write the tile's rows of the output:
+// thread -> (column, 4 channels); splits are summed in order.  ACROSS: the partial results were
+// written by other blocks of the running kernel (device-scope loads); otherwise by a kernel before.
+template <bool ACROSS>
+__device__ __forceinline__ void merge_splits(const float* __restrict__ base, int nsplit, int r, int ct, int kvh, int g,
+                                             const int* __restrict__ cu_q, bf16_t* __restrict__ out, int nq) {
+  const int q0 = cu_q[r], qlen = cu_q[r + 1] - q0;
+  for (int idx = threadIdx.x; idx < 16 * (HD / 4); idx += blockDim.x) {
+    const int col = idx / (HD / 4), d = (idx - col * (HD / 4)) * 4;
+    const int colg = ct * 16 + col;
+    const int i = colg / g, gh = colg - i * g;
+    if (i >= qlen) continue;
+    auto ld = [&](const float* p) { return ACROSS ? load_device_scope(p) : *p; };
+    // Eight splits at a time: their 48 values are asked for together (one trip to memory, not one
+    // per split), then folded into the running sums against the running maximum, in split order.
+    constexpr int AT_ONCE = 8;
+    float m = -INFINITY, den = 0.f;
+    float4 num = {0.f, 0.f, 0.f, 0.f};
+    for (int s0 = 0; s0 < nsplit; s0 += AT_ONCE) {
+      float pm[AT_ONCE], pl[AT_ONCE];
+      float4 pn[AT_ONCE];
+#pragma unroll
+      for (int j = 0; j < AT_ONCE; ++j) {
+        const int s = s0 + j < nsplit ? s0 + j : nsplit - 1;   // beyond the last: read it again, weight 0 below
+        const float* p = base + (size_t)s * PART_STRIDE + col * PART_COLS;
+        pm[j] = ld(p + HD);
+        pl[j] = ld(p + HD + 1);
+        pn[j] = float4{ld(p + d), ld(p + d + 1), ld(p + d + 2), ld(p + d + 3)};
+      }
+      float m_new = m;
+#pragma unroll
+      for (int j = 0; j < AT_ONCE; ++j)
+        if (s0 + j < nsplit) m_new = fmaxf(m_new, pm[j]);
+      const float keep = (m == -INFINITY) ? 0.f : exp2f(m - m_new);
+      num.x *= keep; num.y *= keep; num.z *= keep; num.w *= keep;
+      den *= keep;
+      m = m_new;
+#pragma unroll
+      for (int j = 0; j < AT_ONCE; ++j) {
+        const float wgt = (s0 + j < nsplit && pm[j] != -INFINITY) ? exp2f(pm[j] - m) : 0.f;
+        num.x += wgt * pn[j].x; num.y += wgt * pn[j].y; num.z += wgt * pn[j].z; num.w += wgt * pn[j].w;
+        den += wgt * pl[j];
+      }
+    }
+    const float inv = 1.0f / den;
+    uint2 wv;
+    wv.x = pack2(num.x * inv, num.y * inv);
+    wv.y = pack2(num.z * inv, num.w * inv);
+    *reinterpret_cast<uint2*>(out + ((size_t)(q0 + i) * nq + kvh * g + gh) * HD + d) = wv;
+  }
+}
+
 __global__ __launch_bounds__(64 * COOP_WAVES) void attn_mfma_coop_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
     const int* __restrict__ bt, int table_width, const int* __restrict__ cu_q, const int* __restrict__ ctx_len,
     const int* __restrict__ tile_req, const int* __restrict__ tile_ct, bf16_t* __restrict__ out,
-    float* __restrict__ scratch, int nq, int nkv, int ps, int window, float scale, int nsplit, int keys_per_split) {
+    float* __restrict__ scratch, int* __restrict__ counters, int nq, int nkv, int ps, int window, float scale,
+    int nsplit, int keys_per_split) {
   __shared__ __attribute__((aligned(16))) float sm[COOP_WAVES][PART_STRIDE];
+  __shared__ int is_last;
   const int tile = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lg = lane >> 4, c = lane & 15;
   const int g = nq / nkv;
@@ -914,10 +983,19 @@ __global__ __launch_bounds__(64 * COOP_WAVES) void attn_mfma_coop_kernel(
     const int q0 = cu_q[r], qlen = cu_q[r + 1] - q0;
     if (nsplit > 1) {
       float* part = scratch + (((size_t)tile * nkv + kvh) * nsplit + split) * PART_STRIDE + (size_t)col * PART_COLS;
-      *reinterpret_cast<float4*>(part + d) = num;
-      if (d == 0) {
-        part[HD] = m;
-        part[HD + 1] = den;
+      if (counters) {   // read by another block of this launch
+        store_device_scope(part + d, num.x); store_device_scope(part + d + 1, num.y);
+        store_device_scope(part + d + 2, num.z); store_device_scope(part + d + 3, num.w);
+        if (d == 0) {
+          store_device_scope(part + HD, m);
+          store_device_scope(part + HD + 1, den);
+        }
+      } else {
+        *reinterpret_cast<float4*>(part + d) = num;
+        if (d == 0) {
+          part[HD] = m;
+          part[HD + 1] = den;
+        }
       }
     } else if (i < qlen) {
       const float inv = 1.0f / den;
@@ -927,38 +1005,29 @@ __global__ __launch_bounds__(64 * COOP_WAVES) void attn_mfma_coop_kernel(
       *reinterpret_cast<uint2*>(out + ((size_t)(q0 + i) * nq + kvh * g + gh) * HD + d) = wv;
     }
   }
+  if (nsplit > 1 && counters) {
+    // every thread's stores have arrived before anyone counts this block in
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      int* count = counters + tile * nkv + kvh;
+      const int before = __hip_atomic_fetch_add(count, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      is_last = before == nsplit - 1;
+      if (is_last) __hip_atomic_store(count, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (is_last)
+      merge_splits<true>(scratch + ((size_t)tile * nkv + kvh) * nsplit * PART_STRIDE, nsplit, r, ct, kvh, g, cu_q, out, nq);
+  }
 }
 
 __global__ void attn_mfma_merge_kernel(const float* __restrict__ scratch, const int* __restrict__ cu_q,
                                        const int* __restrict__ tile_req, const int* __restrict__ tile_ct,
                                        bf16_t* __restrict__ out, int nq, int nkv, int nsplit) {
-  // one block per (tile, kv head); thread -> (column, 4 channels); splits are summed in order
-  const int tile = blockIdx.x, kvh = blockIdx.y, g = nq / nkv;
-  const int r = tile_req[tile], ct = tile_ct[tile];
-  const int q0 = cu_q[r], qlen = cu_q[r + 1] - q0;
-  const float* base = scratch + ((size_t)tile * nkv + kvh) * nsplit * PART_STRIDE;
-  for (int idx = threadIdx.x; idx < 16 * (HD / 4); idx += blockDim.x) {
-    const int col = idx / (HD / 4), d = (idx - col * (HD / 4)) * 4;
-    const int colg = ct * 16 + col;
-    const int i = colg / g, gh = colg - i * g;
-    if (i >= qlen) continue;
-    float m = -INFINITY;
-    for (int s = 0; s < nsplit; ++s) m = fmaxf(m, base[(size_t)s * PART_STRIDE + col * PART_COLS + HD]);
-    float4 num = {0.f, 0.f, 0.f, 0.f};
-    float den = 0.f;
-    for (int s = 0; s < nsplit; ++s) {
-      const float* p = base + (size_t)s * PART_STRIDE + col * PART_COLS;
-      const float wgt = (p[HD] == -INFINITY) ? 0.f : exp2f(p[HD] - m);
-      const float4 a = *reinterpret_cast<const float4*>(p + d);
-      num.x += wgt * a.x; num.y += wgt * a.y; num.z += wgt * a.z; num.w += wgt * a.w;
-      den += wgt * p[HD + 1];
-    }
-    const float inv = 1.0f / den;
-    uint2 wv;
-    wv.x = pack2(num.x * inv, num.y * inv);
-    wv.y = pack2(num.z * inv, num.w * inv);
-    *reinterpret_cast<uint2*>(out + ((size_t)(q0 + i) * nq + kvh * g + gh) * HD + d) = wv;
-  }
+  // one block per (tile, kv head)
+  const int tile = blockIdx.x, kvh = blockIdx.y;
+  merge_splits<false>(scratch + ((size_t)tile * nkv + kvh) * nsplit * PART_STRIDE, nsplit, tile_req[tile], tile_ct[tile],
+                      kvh, nq / nkv, cu_q, out, nq);
 }
 
 static int check_common(int num_tiles, int nq, int nkv, int ps, int table_width) {
@@ -1009,8 +1078,8 @@ extern "C" long long qvl_attn_mfma_scratch_floats(int num_tiles, int nkv, int ns
 
 static int launch_coop(const void* q, const void* kc, const void* vc, const void* bt, int table_width,
                        const void* cu_q, const void* ctx_len, const void* tile_req, const void* tile_ct,
-                       int num_tiles, void* out, void* scratch, int nq, int nkv, int ps, int window, float scale,
-                       int nsplit, int keys_per_split, hipStream_t stream) {
+                       int num_tiles, void* out, void* scratch, void* counters, int nq, int nkv, int ps, int window,
+                       float scale, int nsplit, int keys_per_split, hipStream_t stream) {
   const int c = check_common(num_tiles, nq, nkv, ps, table_width);
   if (c >= 0) return c;
   if (nsplit <= 0 || nsplit > 65535 || (nsplit > 1 && (keys_per_split <= 0 || keys_per_split % 32 || !scratch)))
@@ -1019,9 +1088,10 @@ static int launch_coop(const void* q, const void* kc, const void* vc, const void
   hipLaunchKernelGGL(attn_mfma_coop_kernel, dim3(num_tiles, nkv, nsplit), dim3(64 * COOP_WAVES), 0, stream,
                      (const bf16_t*)q, (const bf16_t*)kc, (const bf16_t*)vc, (const int*)bt, table_width,
                      (const int*)cu_q, (const int*)ctx_len, (const int*)tile_req, (const int*)tile_ct, (bf16_t*)out,
-                     (float*)scratch, nq, nkv, ps, window, scale, nsplit, keys_per_split);
+                     (float*)scratch, nsplit > 1 ? (int*)counters : nullptr, nq, nkv, ps, window, scale, nsplit,
+                     keys_per_split);
   if (hipGetLastError() != hipSuccess) return QVL_ERR_LAUNCH;
-  if (nsplit > 1)
+  if (nsplit > 1 && !counters)
     hipLaunchKernelGGL(attn_mfma_merge_kernel, dim3(num_tiles, nkv), dim3(256), 0, stream, (const float*)scratch,
                        (const int*)cu_q, (const int*)tile_req, (const int*)tile_ct, (bf16_t*)out, nq, nkv, nsplit);
   return qvl_launch_status();
@@ -1031,8 +1101,21 @@ extern "C" int qvl_attn_mfma_coop(const void* q, const void* kc, const void* vc,
                                   const void* cu_q, const void* ctx_len, const void* tile_req, const void* tile_ct,
                                   int num_tiles, void* out, void* scratch, int nq, int nkv, int ps, int window,
                                   float scale, int nsplit, int keys_per_split, hipStream_t stream) {
-  return launch_coop(q, kc, vc, bt, table_width, cu_q, ctx_len, tile_req, tile_ct, num_tiles, out, scratch, nq, nkv,
-                     ps, window, scale, nsplit, keys_per_split, stream);
+  return launch_coop(q, kc, vc, bt, table_width, cu_q, ctx_len, tile_req, tile_ct, num_tiles, out, scratch, nullptr, nq,
+                     nkv, ps, window, scale, nsplit, keys_per_split, stream);
+}
+
+// The same with the splits merged inside the one kernel, by the block of each (tile, kv head) that
+// finishes last.  counters: num_tiles * nkv ints, zero before the launch; the launch leaves them at
+// zero.  Launches that share counters or scratch must not overlap.
+extern "C" int qvl_attn_mfma_coop_merged(const void* q, const void* kc, const void* vc, const void* bt, int table_width,
+                                         const void* cu_q, const void* ctx_len, const void* tile_req,
+                                         const void* tile_ct, int num_tiles, void* out, void* scratch, void* counters,
+                                         int nq, int nkv, int ps, int window, float scale, int nsplit,
+                                         int keys_per_split, hipStream_t stream) {
+  if (nsplit > 1 && !counters) return QVL_ERR_SHAPE;
+  return launch_coop(q, kc, vc, bt, table_width, cu_q, ctx_len, tile_req, tile_ct, num_tiles, out, scratch, counters, nq,
+                     nkv, ps, window, scale, nsplit, keys_per_split, stream);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1089,6 +1172,6 @@ extern "C" int qvl_attn_mfma_coop_static(const void* q, const void* kc, const vo
   if (!ptr) return err;
   // Every (tile, head, split) block writes all of its part before the merge kernel reads it, so
   // nothing of the array has to start at zero, whatever the call before left there.
-  return launch_coop(q, kc, vc, bt, table_width, cu_q, ctx_len, tile_req, tile_ct, num_tiles, out, ptr, nq, nkv, ps,
-                     window, scale, nsplit, keys_per_split, stream);
+  return launch_coop(q, kc, vc, bt, table_width, cu_q, ctx_len, tile_req, tile_ct, num_tiles, out, ptr, nullptr, nq, nkv,
+                     ps, window, scale, nsplit, keys_per_split, stream);
 }

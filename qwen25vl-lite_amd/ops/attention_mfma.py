@@ -20,8 +20,10 @@ __all__ = ["try_attention", "supports", "tiles_for", "plan_splits"]
 _c_int, _c_float, _c_ptr = ctypes.c_int, ctypes.c_float, ctypes.c_void_p
 _MAX_HD = 256
 TARGET_BLOCKS = 512        # from here on a wave per tile fills the 256 compute units
-FILL_BLOCKS = 256          # with fewer cooperative blocks than this, long contexts are split
-MIN_KEYS_PER_SPLIT = 1024  # a split is worth a second kernel only above this many keys
+FILL_BLOCKS = 256          # with fewer cooperative blocks than this, contexts are split among blocks
+MIN_KEYS_PER_SPLIT = 256   # the eight waves of a block then have one 32-key block each: a wave has one block's
+                           # loads in flight at a time, so a split shorter than this only adds partial results
+MERGE_COUNTERS = 1 << 16   # (tile, kv head) pairs whose splits one launch can merge by itself
 ALONE_KEYS = 4096          # decoded tokens beside prompt portions get a launch of their own from this context on
 WIDE_WALKS = 768           # the kind of the kernel whose waves carry three column tiles: from this many walks on
 WIDE_BLOCKS = 150_000      # ... that have this many 32-key blocks to walk between them
@@ -74,14 +76,26 @@ def plan_splits(num_tiles: int, nkv: int, max_ctx: int) -> Tuple[str, int, int]:
     if blocks >= TARGET_BLOCKS:
         return "tile", 1, 0
     want = (FILL_BLOCKS + blocks - 1) // blocks
-    nsplit = max(1, min(want, max_ctx // MIN_KEYS_PER_SPLIT))
+    nsplit = max(1, min(want, (max_ctx + MIN_KEYS_PER_SPLIT - 1) // MIN_KEYS_PER_SPLIT))
     if nsplit == 1:
         return "coop", 1, 0
-    per = ((max_ctx + 31 + nsplit - 1) // nsplit + 31) // 32 * 32
+    per = ((max_ctx + nsplit - 1) // nsplit + 31) // 32 * 32
+    # splits begin at a multiple of 32 at or below the first key a tile sees: up to 31 keys more
     return "coop", (max_ctx + 31 + per - 1) // per, per
 
 
 _queues = {}
+_merge_counters = {}
+
+
+def _counters(device: torch.device) -> torch.Tensor:
+    """Per device: the counters by which the blocks of a split attention find out which of them
+    finishes last and merges.  As with the work queues, a launch finds them at zero and leaves
+    them at zero, and launches on one device must follow each other on one stream."""
+    key = torch.device(device).index or 0
+    if key not in _merge_counters:
+        _merge_counters[key] = torch.zeros(MERGE_COUNTERS, dtype=torch.int32, device=device)
+    return _merge_counters[key]
 
 
 def _work_queue(device: torch.device):
@@ -200,6 +214,19 @@ def try_attention(q, k_cache, v_cache, block_table, step, num_q_heads: int, wind
             floats = _fn("attention_mfma", "qvl_attn_mfma_scratch_floats", [_c_int] * 3, defines)
             floats.restype = ctypes.c_longlong
             scratch = torch.empty(int(floats(num_tiles, nkv, nsplit)), dtype=torch.float32, device=q.device)
+        if nsplit > 1 and num_tiles * nkv <= MERGE_COUNTERS:
+            # the block of each (tile, head) that finishes last merges the splits: one launch
+            counters = _counters(q.device)
+            fn = _fn("attention_mfma", "qvl_attn_mfma_coop_merged",
+                     [_c_ptr] * 4 + [_c_int] + [_c_ptr] * 4 + [_c_int, _c_ptr, _c_ptr, _c_ptr] + [_c_int] * 4
+                     + [_c_float, _c_int, _c_int, _c_ptr], defines)
+            code = fn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(step.cu_q),
+                      _ptr(step.ctx_len), _ptr(tile_req), _ptr(tile_ct), num_tiles, _ptr(out), _ptr(scratch),
+                      _ptr(counters), nq, nkv, ps, int(window or 0), float(scale), nsplit, per, _stream())
+            if code:
+                counters.zero_()
+            _check(code, "paged_attention (matrix cores, shared tiles, merged)")
+            return
         fn = _fn("attention_mfma", "qvl_attn_mfma_coop",
                  [_c_ptr] * 4 + [_c_int] + [_c_ptr] * 4 + [_c_int, _c_ptr, _c_ptr] + [_c_int] * 4
                  + [_c_float, _c_int, _c_int, _c_ptr], defines)

@@ -183,18 +183,21 @@ def test_paged_attention_generic(dtype, nq, nkv, hd, window, ps):
     assert torch.allclose(out.float().cpu(), c["want"], **tol), (out.float().cpu() - c["want"]).abs().max()
 
 
-@pytest.mark.parametrize("split", ["tile", "tile_two_groups", "coop", "coop_split"])
+@pytest.mark.parametrize("split", ["tile", "tile_two_groups", "coop", "coop_split", "coop_split_two_kernels"])
 @pytest.mark.parametrize("nq, nkv, hd, window, ps", [(*s, 16) for s in ATTN_SHAPES if s[2] % 16 == 0]
                          + [s for s in PAGE_SIZES if s[2] % 16 == 0])
 def test_paged_attention_matrix_cores(nq, nkv, hd, window, ps, split, monkeypatch):
     """The matrix-core kernels on the same case: blocks that own several tiles and share the keys
     through LDS (one group of waves, or two that take the key blocks in turn and merge), the waves
-    of a block sharing one tile, and the keys further split among blocks."""
+    of a block sharing one tile, and the keys further split among blocks, whose partial results the
+    last block to finish merges (or a second kernel, for callers without counters)."""
     from qwen25vl_lite_amd.ops import attention_mfma
     from qwen25vl_lite_amd.parts import StepContext
     c = _attention_case(torch.bfloat16, nq, nkv, hd, window, ps=ps)
     plan = {"tile": ("tile", 1, 0), "tile_two_groups": ("tile", 1, 0), "coop": ("coop", 1, 0),
-            "coop_split": ("coop", 6, 64)}[split]
+            "coop_split": ("coop", 6, 64), "coop_split_two_kernels": ("coop", 6, 64)}[split]
+    if split == "coop_split_two_kernels":
+        monkeypatch.setattr(attention_mfma, "MERGE_COUNTERS", 0)
     groups = {"tile": 1, "tile_two_groups": 2}.get(split)
     if groups == 2 and hd > 128:
         pytest.skip("two groups of waves are built for head sizes up to 128")
@@ -213,6 +216,12 @@ def test_paged_attention_matrix_cores(nq, nkv, hd, window, ps, split, monkeypatc
     assert out is not None
     err = (out.float().cpu() - c["want"]).abs().max()
     assert torch.allclose(out.float().cpu(), c["want"], atol=1.5e-2, rtol=2e-2), err
+    if split == "coop_split":
+        # the counters are back at zero, and a second launch right behind the first finds them so
+        again = attention_mfma.try_attention(c["q"], c["kc"], c["vc"], c["table"], step, nq, window, c["scale"])
+        assert torch.equal(again, out)
+        torch.cuda.synchronize()
+        assert int(attention_mfma._counters(c["q"].device).abs().sum()) == 0
 
 
 @pytest.mark.parametrize("nq, nkv, hd, window", [(14, 2, 128, None), (6, 2, 48, 100)])
@@ -225,7 +234,7 @@ def test_mixed_step_with_few_long_decoded_tokens(nq, nkv, hd, window, monkeypatc
     from qwen25vl_lite_amd.parts import StepContext
     lens, qlens = (333, 300, 17, 280), (40, 1, 17, 1)
     c = _attention_case(torch.bfloat16, nq, nkv, hd, window, lens, qlens)
-    monkeypatch.setattr(attention_mfma, "TARGET_BLOCKS", 1)
+    monkeypatch.setattr(attention_mfma, "TARGET_BLOCKS", 8)    # the two decoded tokens make 4 blocks, the portions 24 or more
     monkeypatch.setattr(attention_mfma, "MIN_KEYS_PER_SPLIT", 64)
     monkeypatch.setattr(attention_mfma, "ALONE_KEYS", 128)
     cu = [0]
@@ -242,7 +251,7 @@ def test_mixed_step_with_few_long_decoded_tokens(nq, nkv, hd, window, monkeypatc
     real = attention_mfma._fn
     monkeypatch.setattr(attention_mfma, "_fn", lambda stem, name, *a, **k: (called.append(name), real(stem, name, *a, **k))[1])
     out = attention_mfma.try_attention(c["q"], c["kc"], c["vc"], c["table"], step, nq, window, c["scale"])
-    assert "qvl_attn_mfma_coop" in called and "qvl_attn_mfma_block" in called
+    assert "qvl_attn_mfma_coop_merged" in called and "qvl_attn_mfma_block" in called
     err = (out.float().cpu() - c["want"]).abs().max()
     assert torch.allclose(out.float().cpu(), c["want"], atol=1.5e-2, rtol=2e-2), err
 

@@ -75,12 +75,14 @@ def test_context_of_the_benchmark_through_the_real_dispatch(sharp_d, tokens, dty
 
     def spy_fn(stem, name, argtypes, defines=None):
         fn = real_fn(stem, name, argtypes, defines)
-        if name not in ("qvl_attn_mfma_block", "qvl_attn_mfma_coop"):
+        if name not in ("qvl_attn_mfma_block", "qvl_attn_mfma_coop", "qvl_attn_mfma_coop_merged"):
             return fn
 
         def launch(*args):
-            # the kernel for few tiles is told into how many ranges the keys are split (argument 17)
-            seen.append((name, dict(defines or {}, **({"nsplit": args[17]} if name.endswith("coop") else {}))))
+            # the kernel for few tiles is told into how many ranges the keys are split (the argument
+            # before the keys per split and the stream)
+            split = {} if name.endswith("block") else {"nsplit": args[-3], "keys": args[-2]}
+            seen.append(("qvl_attn_mfma_coop" if "coop" in name else name, dict(defines or {}, **split)))
             return fn(*args)
         return launch
 
@@ -118,12 +120,14 @@ def test_context_of_the_benchmark_through_the_real_dispatch(sharp_d, tokens, dty
     assert len(calls(0, "qvl_attn_mfma_block")) == layers and all("BLK_CT" not in d for d in calls(0, "qvl_attn_mfma_block"))
     assert len(calls(1, "qvl_attn_mfma_block")) == layers and all(d.get("BLK_CT") == 3 for d in calls(1, "qvl_attn_mfma_block"))
     # single tokens over 8,280 keys: the keys split among blocks at the real limit of keys per split
-    assert attention_mfma.MIN_KEYS_PER_SPLIT == 1024 and attention_mfma.ALONE_KEYS == 4096
+    assert attention_mfma.MIN_KEYS_PER_SPLIT == 256 and attention_mfma.ALONE_KEYS == 4096
     for i in range(3, 7):
-        assert calls(i, "qvl_attn_mfma_block") == [] and splits(i) == [8] * layers
+        assert calls(i, "qvl_attn_mfma_block") == [] and splits(i) == [33] * layers
+        assert all(d["keys"] == 256 for d in calls(i, "qvl_attn_mfma_coop"))
     # a decoded token with a long context beside a portion: a launch of its own for it, split, and one for the portion
     for i in (7, 8):
-        assert calls(i, "qvl_attn_mfma_block") == [] and splits(i) == [1] * layers + [8] * layers
+        assert calls(i, "qvl_attn_mfma_block") == [] and len(splits(i)) == 2 * layers
+        assert all(n <= 4 for n in splits(i)[:layers]) and splits(i)[layers:] == [33] * layers
     # both decode: one launch, split by the longer context
-    assert calls(9, "qvl_attn_mfma_block") == [] and splits(9) == [8] * layers
+    assert calls(9, "qvl_attn_mfma_block") == [] and len(splits(9)) == layers and all(n >= 29 for n in splits(9))
 
