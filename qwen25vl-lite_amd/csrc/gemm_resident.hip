@@ -11,15 +11,23 @@
 // Wave w covers the 256 values of K from 256 w on, as the A operand (W rows) and B operand (X
 // rows) of v_mfma_f32_16x16x32_bf16; the 16 waves' sums meet in LDS and are added in wave order.
 // Up to 16 rows of X are one column tile of the matrix instruction; 17 to 32 rows are two (MT = 2):
-// every W fragment that is loaded is multiplied with both.  33 to 64 rows are four (MT = 4): they
-// fit neither the registers nor LDS, so X is not resident: for every tile of W each wave reads its
-// columns of all rows of X again (from L2: four times the bytes of the tile's W), and a norm is
-// not folded in (the host hands over normalised rows).
+// every W fragment that is loaded is multiplied with both.  More rows are spread over teams of
+// blocks (below).
 // If K fits one pass (K <= 4096) the X operand stays in registers (the second column tile, if
 // there is one, in LDS, which takes K <= 32 * XHI_STEPS) for all of the block's tiles; W comes
-// through three half-tile buffers that go round, so that the next tile and a half are on their way
-// while a tile is multiplied and its sums are merged.  A longer K is walked in passes of 4096 that
-// take their turns in the same rotation (X is then read again for every pass).
+// through two half-tile buffers, each asked for again the moment its half is multiplied, so that
+// the next tile is on its way while a tile is multiplied and its sums are merged.  (A third buffer
+// fits the registers only if the compiler keeps every load in the place it was written; it does
+// not, and spills cost more than the deeper stream gains.)  A longer K is walked in passes of 4096
+// that take their turns in the same rotation (X is then read again for every pass).
+//
+// Every load of the stream goes through a buffer descriptor (buffer_load with a byte offset that
+// the hardware checks against the buffer's size): a lane that has nothing to load (a row beyond
+// the tile, a column beyond K, a tile beyond the last) asks at an offset past the end and gets
+// zeros without any traffic.  So no load sits inside a branch, every wave issues the same loads
+// in the same order whatever its data, and the compiler can count exactly how many younger loads
+// may stay in flight at each wait (a load inside a branch costs a wait for everything: the
+// counter only says how many loads are outstanding, and the loads come back in order).
 //
 // What is folded in:
 //   prologue  PRO_NORM      X = rmsnorm(H) * w, from the float32 residual H (statistics in float32,
@@ -38,6 +46,40 @@ typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+// An offset no buffer reaches: what is loaded there is zero.  Buffers stay below it (the host checks).
+#define PAST_END 0xffffff00u
+#define BUFFER_LIMIT 0xffffff00ull
+
+__device__ __forceinline__ rsrc_t buffer_of(const void* p, unsigned long long bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, p ? (int)(uint32_t)bytes : 0, 0x00020000);
+}
+// `fixed` is a compile-time part of the offset: it rides in the instruction, the lanes' part in one register.
+__device__ __forceinline__ u32x4_t buffer_load16(rsrc_t r, uint32_t byte_offset, int fixed = 0) {
+  return __builtin_amdgcn_raw_buffer_load_b128(r, byte_offset, fixed, 0);
+}
+__device__ __forceinline__ float buffer_load_f32(rsrc_t r, uint32_t byte_offset) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, byte_offset, 0, 0));
+}
+
+#define HOLD_ORDER() __builtin_amdgcn_sched_barrier(0)   // nothing is scheduled across this point
+
+#ifdef QVL_TIMELINE
+// Measurement aid (never compiled into the package's library): every block's first wave stamps the
+// device's 100 MHz clock at a few places into a buffer set by qvl_gemm_resident_timeline().
+static unsigned long long* timeline_buffer = nullptr;
+extern "C" void qvl_gemm_resident_timeline(void* p) { timeline_buffer = (unsigned long long*)p; }
+#define STAMP(i)                                                                                    \
+  do {                                                                                              \
+    if (p.timeline && threadIdx.x == 0) p.timeline[blockIdx.x * 8 + (i)] = __builtin_amdgcn_s_memrealtime(); \
+  } while (0)
+#else
+#define STAMP(i)
+#endif
+
+#ifndef W_RING
+#define W_RING 2   // half-step buffers of W that go round
+#endif
 #define RW 16   // waves per block
 #define RK 8    // 32-wide K steps per wave and pass
 #define PASS_K (RW * RK * 32)
@@ -78,6 +120,9 @@ struct ResidentArgs {
   // is cut into `parts` tiles of `pairs` gate rows and their up rows, so that the last round of
   // tiles is as even as the rounds before it
   int whole_tiles, parts, pairs;
+#ifdef QVL_TIMELINE
+  unsigned long long* timeline;
+#endif
 };
 
 __device__ __forceinline__ bf16x8_t load8(const bf16_t* p) {
@@ -97,8 +142,7 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
   constexpr int COLS = 16 * MT;   // rows of X the block carries
   // MT = 1: two buffers, a tile's sums are read while the next tile's are written.  MT = 2: one
   // (LDS also holds the second column tile of X), and the norm weights borrow it before the first tile.
-  static_assert(MT == 1 || MT == 2 || MT == 4, "one, two or four column tiles");
-  static_assert(MT != 4 || PRO == PRO_PLAIN, "with four column tiles the rows arrive normalised");
+  static_assert(MT == 1 || MT == 2, "one or two column tiles");
   __shared__ __attribute__((aligned(16))) float red[MT == 1 ? 2 : 1][RW][16 * COLS];
   __shared__ float rowsq[RW][16];
   __shared__ __attribute__((aligned(16))) float gains_own[(PRO == PRO_NORM && MT == 1) ? RW : 1][RK * 32];
@@ -106,6 +150,19 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
   float (*gains)[RK * 32] = MT == 1 ? gains_own : reinterpret_cast<float (*)[RK * 32]>(&red[0][0][0]);  // norm weights of each wave's columns
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, lg = lane >> 4, r = lane & 15;
   const int k_lane = wave * RK * 32 + 8 * lg;  // first K index of this lane within a pass
+  STAMP(0);
+  // how many of this lane's 32-wide steps of the pass that starts at k0 begin inside K (K is a
+  // multiple of 8, as is every lane's first index: a step lies inside K or outside)
+  auto steps_inside = [&](int k0) { return (p.K - k0 - k_lane + 31) >> 5; };
+  // what the kernel reads, each behind a descriptor that knows its size (a null pointer: size 0)
+  const rsrc_t w_buf = buffer_of(p.W, ((unsigned long long)(p.N - 1) * p.ldw + p.K) * 2);
+  const rsrc_t x_buf = buffer_of(p.X, ((unsigned long long)(p.M - 1) * p.ldx + p.K) * 2);
+  const rsrc_t h_buf = buffer_of(p.H, ((unsigned long long)(p.M - 1) * p.ldh + p.K) * 4);
+  const rsrc_t gain_buf = buffer_of(p.norm_w, (unsigned long long)p.K * 4);
+  const rsrc_t bias_buf = buffer_of(p.bias, (unsigned long long)p.N * 4);
+  const rsrc_t old_buf = buffer_of(EPI == EPI_RESIDUAL ? p.out : nullptr, ((unsigned long long)(p.M - 1) * p.ldo + p.N) * 4);
+  const rsrc_t cs_buf = buffer_of(p.cs, (unsigned long long)p.M * p.hd * 4);
+  const rsrc_t slot_buf = buffer_of(p.slot, (unsigned long long)p.M * 4);
   // Workgroups go to the XCDs in turn, so blocks b, b + 8, b + 16, ... share an XCD: consecutive
   // ones of them form a team.
   int team = blockIdx.x, teams = gridDim.x, m0 = 0;   // m0: this block's first row of X
@@ -125,33 +182,29 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
     const bool m_ok = row < p.M;
     if (PRO == PRO_PLAIN) {
       first_w();   // W first: it is the long wait
-      const bf16_t* xrow = p.X + (size_t)(m_ok ? row : 0) * p.ldx;
+      const uint32_t at = m_ok ? ((uint32_t)row * p.ldx + k0 + k_lane) * 2 : PAST_END;
+      const int inside = steps_inside(k0);
 #pragma unroll
-      for (int u = 0; u < RK; ++u) {
-        const int k = k0 + k_lane + u * 32;
-        xb[u] = (m_ok && k < p.K) ? load8(xrow + k) : zero8();
-      }
+      for (int u = 0; u < RK; ++u)
+        xb[u] = __builtin_bit_cast(bf16x8_t, buffer_load16(x_buf, u < inside ? at : PAST_END, u * 64));
     } else {
       // rmsnorm of the float32 rows: this pass covers all of K (ONE_PASS), so the block's waves
       // hold whole rows between them.  Loads return in the order they are issued: the rows and
       // the norm weights are asked for first and W (by first_w) right behind them, so the
       // statistics and the scaling run while W is still on its way.  A lane fetches 4 of its
       // wave's 256 norm weights; they reach the lanes that need them through LDS.
-      const float* hrow = p.H + (size_t)(m_ok ? row : 0) * p.ldh;
+      const uint32_t at = m_ok ? ((uint32_t)row * p.ldh + k_lane) * 4 : PAST_END;
+      const int inside = steps_inside(0);
       float4 v[RK][2];
 #pragma unroll
       for (int u = 0; u < RK; ++u) {
-        const int k = k_lane + u * 32;
-        if (m_ok && k < p.K) {
-          v[u][0] = *reinterpret_cast<const float4*>(hrow + k);
-          v[u][1] = *reinterpret_cast<const float4*>(hrow + k + 4);
-        } else {
-          v[u][0] = v[u][1] = float4{0.f, 0.f, 0.f, 0.f};
-        }
+        const uint32_t o = u < inside ? at : PAST_END;
+        v[u][0] = __builtin_bit_cast(float4, buffer_load16(h_buf, o, u * 128));
+        v[u][1] = __builtin_bit_cast(float4, buffer_load16(h_buf, o, u * 128 + 16));
       }
       const int kg = wave * RK * 32 + 4 * lane;
-      float4 g4 = {0.f, 0.f, 0.f, 0.f};
-      if (!again && kg < p.K) g4 = *reinterpret_cast<const float4*>(p.norm_w + kg);
+      // beyond K the descriptor's own size gives zeros (K is a multiple of 8, kg of 4)
+      const float4 g4 = __builtin_bit_cast(float4, buffer_load16(gain_buf, again ? PAST_END : (uint32_t)kg * 4));
       first_w();
       float ss = 0.f;
 #pragma unroll
@@ -160,18 +213,20 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
               v[u][1].x * v[u][1].x + v[u][1].y * v[u][1].y + v[u][1].z * v[u][1].z + v[u][1].w * v[u][1].w;
       ss += __shfl_xor(ss, 16, QVL_WAVE);
       ss += __shfl_xor(ss, 32, QVL_WAVE);
+      asm volatile("s_nop 0" ::"v"(ss));
+      STAMP(6);   // this wave's rows have arrived
       if (again) __syncthreads();   // the other column tile's statistics have been read
       if (lg == 0) rowsq[wave][r] = ss;
       if (!again) *reinterpret_cast<float4*>(&gains[wave][4 * lane]) = g4;
       __syncthreads();
+      STAMP(7);   // every wave's have
       float total = 0.f;
 #pragma unroll
       for (int w = 0; w < RW; ++w) total += rowsq[w][r];
       const float rs = 1.0f / sqrtf(total / (float)p.K + p.eps);
 #pragma unroll
       for (int u = 0; u < RK; ++u) {
-        const int k = k_lane + u * 32;
-        if (k < p.K) {
+        if (u < inside) {
           const float4 g0 = *reinterpret_cast<const float4*>(&gains[wave][8 * lg + u * 32]);
           const float4 g1 = *reinterpret_cast<const float4*>(&gains[wave][8 * lg + u * 32 + 4]);
           u32x4_t o = {pack2((v[u][0].x * rs) * g0.x, (v[u][0].y * rs) * g0.y),
@@ -204,14 +259,14 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
   };
   // steps u0 .. u0 + n - 1 of a tile's W operand
   auto load_w_part = [&](int tile, int k0, int u0, int n, bf16x8_t* a) {
-    const int row = w_row(tile, r);
+    // a tile beyond the last has no rows: all of its loads are asked for past the end
+    const int row = tile < p.ntiles ? w_row(tile, r) : -1;
     const bool row_ok = r < tile_rows(tile) && row >= 0 && row < p.N;
-    const bf16_t* wrow = p.W + (size_t)(row_ok ? row : 0) * p.ldw;
+    const uint32_t at = row_ok ? ((uint32_t)row * p.ldw + k0 + k_lane) * 2 : PAST_END;
+    const int inside = steps_inside(k0);
 #pragma unroll
-    for (int u = 0; u < n; ++u) {
-      const int k = k0 + k_lane + (u0 + u) * 32;
-      a[u] = (row_ok && k < p.K) ? load8(wrow + k) : zero8();
-    }
+    for (int u = 0; u < n; ++u)
+      a[u] = __builtin_bit_cast(bf16x8_t, buffer_load16(w_buf, u0 + u < inside ? at : PAST_END, (u0 + u) * 64));
   };
   auto load_w = [&](int tile, int k0, bf16x8_t* a) { load_w_part(tile, k0, 0, RK, a); };
   // What the epilogue of a tile reads from memory, for the element (m, nl) this thread finishes.
@@ -227,16 +282,22 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
     e.bias = e.old = 0.f;
     e.cs = float2{1.f, 0.f};
     e.slot = -1;
-    if (threadIdx.x >= 16 * COLS || EPI == EPI_SWIGLU) return e;
-    const int m = m0 + (threadIdx.x >> 4), nl = threadIdx.x & 15, n = w_row(tile, nl);
-    if (m >= p.M || nl >= tile_rows(tile) || n >= p.N) return e;
-    if (p.bias) e.bias = p.bias[n];
-    if (EPI == EPI_RESIDUAL) e.old = reinterpret_cast<const float*>(p.out)[(size_t)m * p.ldo + n];
+    if (EPI == EPI_SWIGLU) return e;
+    // Every thread asks, the ones without an element past the end (and gets zeros): the same loads
+    // on every path.  The waves beyond the first 16 COLS threads have no element at all.
+    const int m = m0 + (threadIdx.x >> 4), nl = threadIdx.x & 15;
+    const int n = tile < p.ntiles ? w_row(tile, nl) : -1;
+    const bool live = threadIdx.x < 16 * COLS && m < p.M && nl < tile_rows(tile) && n >= 0 && n < p.N;
+    e.bias = buffer_load_f32(bias_buf, live ? (uint32_t)n * 4 : PAST_END);
+    if (EPI == EPI_RESIDUAL) e.old = buffer_load_f32(old_buf, live ? ((uint32_t)m * p.ldo + n) * 4 : PAST_END);
     if (EPI == EPI_ROPE) {
-      const int head = n / p.hd, d = n - head * p.hd, half = p.hd >> 1;
-      if (head < p.nq + p.nkv)
-        e.cs = *reinterpret_cast<const float2*>(p.cs + ((size_t)m * half + (d < half ? d : d - half)) * 2);
-      if (head >= p.nq) e.slot = p.slot[m];
+      const int head = live ? n / p.hd : 0, d = n - head * p.hd, half = p.hd >> 1;
+      const bool turns = live && head < p.nq + p.nkv;
+      const uint32_t at = turns ? ((uint32_t)m * half + (d < half ? d : d - half)) * 8 : PAST_END;
+      e.cs = float2{buffer_load_f32(cs_buf, at), buffer_load_f32(cs_buf, at + 4)};
+      if (!turns) e.cs = float2{1.f, 0.f};
+      const int slot = __builtin_bit_cast(int, buffer_load_f32(slot_buf, (live && head >= p.nq) ? (uint32_t)m * 4 : PAST_END));
+      e.slot = (live && head >= p.nq) ? slot : -1;
     }
     return e;
   };
@@ -325,51 +386,19 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
   auto load_x_half = [&](int k0, int half, bf16x8_t* xb) {
     const int row = m0 + r;
     const bool m_ok = row < p.M;
-    const bf16_t* xrow = p.X + (size_t)(m_ok ? row : 0) * p.ldx;
+    const uint32_t at = m_ok ? ((uint32_t)row * p.ldx + k0 + k_lane) * 2 : PAST_END;
+    const int inside = steps_inside(k0);
 #pragma unroll
     for (int i = 0; i < RK / 2; ++i) {
-      const int u = half * (RK / 2) + i, k = k0 + k_lane + u * 32;
-      xb[u] = (m_ok && k < p.K) ? load8(xrow + k) : zero8();
+      const int u = half * (RK / 2) + i;
+      xb[u] = __builtin_bit_cast(bf16x8_t, buffer_load16(x_buf, u < inside ? at : PAST_END, u * 64));
     }
-  };
-  // MT = 4: the X operands of the pass that starts at k0 come from memory (L2) for every tile, two
-  // steps of a column tile at a time through two small buffers that take turns, so that the next
-  // loads are on their way while these are multiplied (and the other waves of the SIMD fill the rest
-  // of the wait).
-  auto product_streamed = [&](const bf16x8_t* a_lo, const bf16x8_t* a_hi, int k0, Acc acc) {
-    constexpr int Q = 2, PARTS = RK / Q, CHUNKS = MT * PARTS;
-    bf16x8_t xs[2][Q];
-    auto load_chunk = [&](int c, bf16x8_t* dst) {
-      const int t = c / PARTS, part = c % PARTS;
-      const int row = m0 + 16 * t + r;
-      const bool m_ok = row < p.M;
-      const bf16_t* xrow = p.X + (size_t)(m_ok ? row : 0) * p.ldx;
-#pragma unroll
-      for (int u = 0; u < Q; ++u) {
-        const int k = k0 + k_lane + (part * Q + u) * 32;
-        dst[u] = (m_ok && k < p.K) ? load8(xrow + k) : zero8();
-      }
-    };
-    load_chunk(0, xs[0]);
-    load_chunk(1, xs[1]);
-#pragma unroll
-    for (int c = 0; c < CHUNKS; ++c) {
-      const int t = c / PARTS, part = c % PARTS;
-#pragma unroll
-      for (int u = 0; u < Q; ++u) {
-        const int step = part * Q + u;
-        const bf16x8_t a = step < RK / 2 ? a_lo[step] : a_hi[step - RK / 2];
-        acc.t[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, xs[c & 1][u], acc.t[t], 0, 0, 0);
-      }
-      if (c + 2 < CHUNKS) load_chunk(c + 2, xs[c & 1]);
-    }
-    return acc;
   };
   Acc zero;
 #pragma unroll
   for (int t = 0; t < MT; ++t) zero.t[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-  if (ONE_PASS || MT == 1 || MT == 4) {
+  if (ONE_PASS || MT == 1) {
     // The block's work is a sequence of steps: every tile of its own, and within a tile every pass
     // over K (one, if X stays resident).  Three half-step buffers of W go round: while a step is
     // multiplied, the first half of the next is on its way; its second half and the first half of
@@ -383,68 +412,67 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
       }
     };
     bf16x8_t xb[RK];
-    bf16x8_t w[3][RK / 2];
+    bf16x8_t w[W_RING][RK / 2];
     int tile = team, pass = 0;
-    if (MT == 4) {
-      if (tile < p.ntiles) {
+    if (MT == 1) {
+      load_x(0, 0, xb, [&] {
         load_w_part(tile, 0, 0, RK / 2, w[0]);
         load_w_part(tile, 0, RK / 2, RK / 2, w[1]);
-      }
-    } else if (MT == 1) {
-      load_x(0, 0, xb, [&] {
-        if (tile < p.ntiles) {
-          load_w_part(tile, 0, 0, RK / 2, w[0]);
-          load_w_part(tile, 0, RK / 2, RK / 2, w[1]);
-        }
       });
     } else {
       // rows 16..31 first, while few registers are taken: each lane keeps its own operands of
       // them in LDS and reads them back itself
       bf16x8_t hi[RK];
-      load_x(1, 0, hi, [&] { if (tile < p.ntiles) load_w_part(tile, 0, 0, RK / 2, w[0]); });
+      load_x(1, 0, hi, [&] { load_w_part(tile, 0, 0, RK / 2, w[0]); });
 #pragma unroll
       for (int u = 0; u < RK; ++u)
         if (hi_live) xhi[(wave * RK + u) * 64 + lane] = __builtin_bit_cast(u32x4_t, hi[u]);
-      load_x(0, 0, xb, [&] { if (tile < p.ntiles) load_w_part(tile, 0, RK / 2, RK / 2, w[1]); }, true);
+      load_x(0, 0, xb, [&] { load_w_part(tile, 0, RK / 2, RK / 2, w[1]); }, true);
       if (PRO == PRO_NORM) __syncthreads();   // the norm weights lie where the first tile's sums go
     }
+    STAMP(1);   // the rows are in their registers, the first tile asked for
     Epi e = epi_load(tile);
+#if W_RING == 3
     {
       int t1 = tile, p1 = 0;
       step_after(t1, p1);
-      if (t1 < p.ntiles) load_w_part(t1, p1 * PASS_K, 0, RK / 2, w[2]);
+      load_w_part(t1, p1 * PASS_K, 0, RK / 2, w[2]);
     }
+#endif
     Acc acc = zero;
     // one step whose halves are in a_lo and a_hi; false: it was the block's last
     // A half buffer is asked for again the moment its steps are multiplied (not after the whole
-    // step): every half then has a whole period, a step and a merge, to arrive in.  Between the
-    // passes of a tile the next rows of X are asked for the same way, each half ahead of the W
-    // half that is needed with it (loads come back in the order they were asked for).
+    // step).  Between the passes of a tile the next rows of X are asked for the same way, each half
+    // ahead of the W half that is needed with it (loads come back in the order they were asked
+    // for).  Every step issues the same loads, a step beyond the block's last one past the end of
+    // the buffers.  With a ring of three half buffers the half that is free takes the first half of
+    // the step after next; with two, each half takes its own part of the next step.
     auto one = [&](bf16x8_t* a_lo, bf16x8_t* a_hi) {
       int tn = tile, pn = pass;
       step_after(tn, pn);
       int ta = tn, pa = pn;
       step_after(ta, pa);
       const bool tile_done = ONE_PASS || pn == 0;
-      Epi e_next = e;
-      if constexpr (MT == 4) {
-        acc = product_streamed(a_lo, a_hi, pass * PASS_K, acc);
-        if (tile_done) e_next = epi_load(tn);
-        if (tn < p.ntiles) load_w_part(tn, pn * PASS_K, RK / 2, RK / 2, a_lo);
-        if (ta < p.ntiles) load_w_part(ta, pa * PASS_K, 0, RK / 2, a_hi);
-      } else {
-        acc = product_part(a_lo, 0, RK / 2, xb, nullptr, acc);
-        if (tn < p.ntiles) {
-          if (!ONE_PASS && MT == 1) load_x_half(pn * PASS_K, 0, xb);
-          load_w_part(tn, pn * PASS_K, RK / 2, RK / 2, a_lo);
-        }
-        acc = product_part(a_hi, RK / 2, RK / 2, xb, nullptr, acc);
-        if (tile_done) e_next = epi_load(tn);
-        if (tn < p.ntiles && !ONE_PASS && MT == 1) load_x_half(pn * PASS_K, 1, xb);
-        if (ta < p.ntiles) load_w_part(ta, pa * PASS_K, 0, RK / 2, a_hi);
-      }
+      // the order below is the order of the instructions: the compiler's scheduler would pull the
+      // loads of later steps ahead of the products and run out of registers for them
+      HOLD_ORDER();
+      acc = product_part(a_lo, 0, RK / 2, xb, nullptr, acc);
+      if (tile == team) { asm volatile("s_nop 0" :: "v"(acc.t[0])); STAMP(2); }   // the first half tile was there
+      HOLD_ORDER();
+      if (!ONE_PASS && MT == 1) load_x_half(pn * PASS_K, 0, xb);
+      load_w_part(tn, pn * PASS_K, W_RING == 3 ? RK / 2 : 0, RK / 2, a_lo);
+      HOLD_ORDER();
+      acc = product_part(a_hi, RK / 2, RK / 2, xb, nullptr, acc);
+      HOLD_ORDER();
+      const Epi e_next = epi_load(tn);
+      if (!ONE_PASS && MT == 1) load_x_half(pn * PASS_K, 1, xb);
+      if (W_RING == 3) load_w_part(ta, pa * PASS_K, 0, RK / 2, a_hi);
+      else load_w_part(tn, pn * PASS_K, RK / 2, RK / 2, a_hi);
+      HOLD_ORDER();
       if (tile_done) {
+        if (tile == team) STAMP(3);   // all of the first tile multiplied
         finish(tile, acc, e);
+        if (tile == team) STAMP(4);   // and merged and written
         acc = zero;
         e = e_next;
       }
@@ -454,9 +482,12 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
     };
     while (tile < p.ntiles) {
       if (!one(w[0], w[1])) break;
+#if W_RING == 3
       if (!one(w[2], w[0])) break;
       if (!one(w[1], w[2])) break;
+#endif
     }
+    STAMP(5);
   } else {
     for (int tile = team; tile < p.ntiles; tile += teams) {
       Acc acc = zero;
@@ -476,7 +507,7 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
 // in the block for all its tiles (one pass over K).  Up to 32 rows one block carries them all.
 // More rows, or 17 to 32 rows with a K too long for the second column tile's place in LDS, are
 // spread over the blocks of a team; a device with too few compute units for teams (fewer than 8
-// per group) falls back on one block that streams X (MT = 4).
+// per group) is refused (mt = 0).
 struct Plan {
   int mt, groups;
   bool one_pass;
@@ -489,7 +520,7 @@ static Plan plan_for(int M, int K, bool norm, int blocks, bool prefer_teams) {
   const int singles = (M + 15) / 16;
   if ((M > 32 || prefer_teams || norm) && blocks >= 8 * singles) return Plan{1, singles, K <= PASS_K};
   if (M <= 32) return Plan{2, 1, false};
-  return Plan{4, 1, K <= PASS_K};
+  return Plan{0, 1, false};
 }
 // the number of teams the plan's grid has: what the tiles are divided among
 static int plan_teams(const Plan& pl, int blocks) { return pl.groups == 1 ? blocks : blocks / (8 * pl.groups) * 8; }
@@ -507,9 +538,6 @@ static int launch(ResidentArgs p, const Plan& pl, int blocks, hipStream_t stream
   } else if (pl.mt == 2) {
     if (pl.one_pass) QVL_GO(true, 2);
     else if constexpr (PRO == PRO_PLAIN) QVL_GO(false, 2);
-  } else if constexpr (PRO == PRO_PLAIN) {
-    if (pl.one_pass) QVL_GO(true, 4);
-    else QVL_GO(false, 4);
   } else {
     return QVL_ERR_LIMIT;
   }
@@ -524,6 +552,16 @@ extern "C" int qvl_gemm_resident_folds_norm(int M, int K, int blocks) {
   const Plan pl = plan_for(M, K, true, blocks, false);
   return pl.one_pass && pl.mt <= 2;
 }
+
+// Whether every operand lies within what a buffer descriptor and a 32-bit byte offset reach.
+static bool fits_descriptors(long long M, long long N, long long K, long long ldw, long long ldx, long long ldh,
+                             long long ldo) {
+  const unsigned long long w = ((N - 1) * ldw + K) * 2ull, x = ((M - 1) * ldx + K) * 2ull,
+                           h = ((M - 1) * ldh + K) * 4ull, o = ((M - 1) * ldo + N) * 4ull;
+  return w < BUFFER_LIMIT && x < BUFFER_LIMIT && h < BUFFER_LIMIT && o < BUFFER_LIMIT;
+}
+// The most bytes a weight matrix may span ((N - 1) ldw + K elements of two bytes).
+extern "C" unsigned long long qvl_gemm_resident_max_weight_bytes() { return BUFFER_LIMIT - 1; }
 
 extern "C" int qvl_gemm_resident_pass_k() { return PASS_K; }
 // the longest K with which 17 to 32 rows stay resident (and with which their norm is folded in)
@@ -542,6 +580,7 @@ extern "C" int qvl_gemm_resident(const void* x, int ldx, const void* h, int ldh,
   if (M > 64) return QVL_ERR_LIMIT;
   if (M > 32 && K > PASS_K) return QVL_ERR_LIMIT;   // teams of more than two keep their rows for a single pass
   if (K <= 0 || K % 8 || ldw % 8 || ldw < K || max_blocks <= 0 || !W || !out) return QVL_ERR_SHAPE;
+  if (!fits_descriptors(M, N, K, ldw, ldx, ldh, ldo)) return QVL_ERR_LIMIT;
   const bool norm = h != nullptr;
   const Plan pl = plan_for(M, K, norm, max_blocks, flags & 1);
   const int teams = plan_teams(pl, max_blocks);
@@ -560,6 +599,9 @@ extern "C" int qvl_gemm_resident(const void* x, int ldx, const void* h, int ldh,
   p.X = (const bf16_t*)x; p.ldx = ldx; p.H = (const float*)h; p.ldh = ldh; p.norm_w = (const float*)norm_w;
   p.eps = eps; p.W = (const bf16_t*)W; p.ldw = ldw; p.bias = (const float*)bias; p.out = out; p.ldo = ldo;
   p.M = M; p.N = N; p.K = K;
+#ifdef QVL_TIMELINE
+  p.timeline = timeline_buffer;
+#endif
   p.cs = nullptr; p.slot = nullptr;
   p.q_out = nullptr; p.kc = nullptr; p.vc = nullptr; p.nq = p.nkv = p.hd = p.ps = 0; p.pair_tiles = 0;
   // as many rounds of tiles as 16-row tiles need, with rows per tile cut down to what fills them evenly
@@ -605,6 +647,8 @@ extern "C" int qvl_gemm_resident_rope(const void* x, int ldx, const void* h, int
   if (M > 64) return QVL_ERR_LIMIT;
   if (M > 32 && K > PASS_K) return QVL_ERR_LIMIT;   // as in qvl_gemm_resident
   if (K <= 0 || K % 8 || ldw % 8 || ldw < K || max_blocks <= 0 || !W || !q_out) return QVL_ERR_SHAPE;
+  if (nq <= 0 || nkv < 0 || hd <= 0) return QVL_ERR_SHAPE;
+  if (!fits_descriptors(M, (nq + 2 * nkv) * hd, K, ldw, ldx, ldh, 0)) return QVL_ERR_LIMIT;
   if (nq <= 0 || nkv < 0 || hd <= 0 || hd % 16 || ps <= 0 || !cs) return QVL_ERR_SHAPE;
   if (nkv > 0 && (!slot || !kc || !vc)) return QVL_ERR_SHAPE;
   const bool norm = h != nullptr;
@@ -620,6 +664,9 @@ extern "C" int qvl_gemm_resident_rope(const void* x, int ldx, const void* h, int
   p.X = (const bf16_t*)x; p.ldx = ldx; p.H = (const float*)h; p.ldh = ldh; p.norm_w = (const float*)norm_w;
   p.eps = eps; p.W = (const bf16_t*)W; p.ldw = ldw; p.bias = (const float*)bias; p.out = nullptr; p.ldo = 0;
   p.M = M; p.N = (nq + 2 * nkv) * hd; p.K = K;
+#ifdef QVL_TIMELINE
+  p.timeline = timeline_buffer;
+#endif
   // query and key heads in tiles of 8 + 8 rows, then the value rows in tiles as small as fills
   // the compute units evenly (36 heads of 128 on 256 units: 256 tiles of 16 and 256 of 2)
   p.pair_tiles = (nq + nkv) * (hd / 16);

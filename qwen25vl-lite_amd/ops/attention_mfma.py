@@ -21,8 +21,8 @@ _c_int, _c_float, _c_ptr = ctypes.c_int, ctypes.c_float, ctypes.c_void_p
 _MAX_HD = 256
 TARGET_BLOCKS = 512        # from here on a wave per tile fills the 256 compute units
 FILL_BLOCKS = 256          # with fewer cooperative blocks than this, contexts are split among blocks
-MIN_KEYS_PER_SPLIT = 256   # the eight waves of a block then have one 32-key block each: a wave has one block's
-                           # loads in flight at a time, so a split shorter than this only adds partial results
+MIN_KEYS_PER_SPLIT = 1024  # merging the splits (stores, a counter and loads that go through to memory) costs a decode
+                           # step about as much as each wave's walk over four more 32-key blocks: shorter splits lose
 MERGE_COUNTERS = 1 << 16   # (tile, kv head) pairs whose splits one launch can merge by itself
 ALONE_KEYS = 4096          # decoded tokens beside prompt portions get a launch of their own from this context on
 WIDE_WALKS = 768           # the kind of the kernel whose waves carry three column tiles: from this many walks on
@@ -76,11 +76,11 @@ def plan_splits(num_tiles: int, nkv: int, max_ctx: int) -> Tuple[str, int, int]:
     if blocks >= TARGET_BLOCKS:
         return "tile", 1, 0
     want = (FILL_BLOCKS + blocks - 1) // blocks
-    nsplit = max(1, min(want, (max_ctx + MIN_KEYS_PER_SPLIT - 1) // MIN_KEYS_PER_SPLIT))
+    nsplit = max(1, min(want, max_ctx // MIN_KEYS_PER_SPLIT))
     if nsplit == 1:
         return "coop", 1, 0
-    per = ((max_ctx + nsplit - 1) // nsplit + 31) // 32 * 32
     # splits begin at a multiple of 32 at or below the first key a tile sees: up to 31 keys more
+    per = ((max_ctx + 31 + nsplit - 1) // nsplit + 31) // 32 * 32
     return "coop", (max_ctx + 31 + per - 1) // per, per
 
 

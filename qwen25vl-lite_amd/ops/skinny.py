@@ -22,6 +22,7 @@ RESIDENT_ROWS = 64       # up to here the resident kernel runs
 ONE_BLOCK_ROWS = 32      # up to here one block carries all rows: beyond, teams of blocks share the weight's
                          # tiles, which pays for the fused q | k | v projection only
 TEAM_LONG_K = 1          # flag: 17 to 32 rows with a long inner size go to a team of two blocks
+_MAX_WEIGHT_BYTES = 0xffffff00   # qvl_gemm_resident_max_weight_bytes() + 1
 _pass_k = None
 _two_tile_k = None
 STORE, RESIDUAL, SWIGLU = 0, 1, 2
@@ -76,6 +77,8 @@ def takes_resident(m: int, k: int, weight: torch.Tensor, *, norm: bool = False) 
     decoder's shapes, K of 8192 and 29568)."""
     if m > RESIDENT_ROWS or k % 8 or weight.dtype != torch.bfloat16 or not _rows_aligned(weight, 8):
         return False
+    if ((weight.shape[0] - 1) * weight.stride(0) + k) * 2 >= _MAX_WEIGHT_BYTES:
+        return False     # the kernel reaches its operands through 32-bit byte offsets
     if norm:
         return folds_norm(m, k, weight.device)
     if m > 32:

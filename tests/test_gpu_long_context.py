@@ -120,14 +120,16 @@ def test_context_of_the_benchmark_through_the_real_dispatch(sharp_d, tokens, dty
     assert len(calls(0, "qvl_attn_mfma_block")) == layers and all("BLK_CT" not in d for d in calls(0, "qvl_attn_mfma_block"))
     assert len(calls(1, "qvl_attn_mfma_block")) == layers and all(d.get("BLK_CT") == 3 for d in calls(1, "qvl_attn_mfma_block"))
     # single tokens over 8,280 keys: the keys split among blocks at the real limit of keys per split
-    assert attention_mfma.MIN_KEYS_PER_SPLIT == 256 and attention_mfma.ALONE_KEYS == 4096
+    per = attention_mfma.MIN_KEYS_PER_SPLIT
+    assert per <= 1024 and attention_mfma.ALONE_KEYS == 4096
+    many = 8280 // per      # as many splits as the limit of keys per split allows: the blocks are few
     for i in range(3, 7):
-        assert calls(i, "qvl_attn_mfma_block") == [] and splits(i) == [33] * layers
-        assert all(d["keys"] == 256 for d in calls(i, "qvl_attn_mfma_coop"))
+        assert calls(i, "qvl_attn_mfma_block") == [] and splits(i) == [many] * layers
+        assert all(per <= d["keys"] < per + 64 for d in calls(i, "qvl_attn_mfma_coop"))
     # a decoded token with a long context beside a portion: a launch of its own for it, split, and one for the portion
     for i in (7, 8):
         assert calls(i, "qvl_attn_mfma_block") == [] and len(splits(i)) == 2 * layers
-        assert all(n <= 4 for n in splits(i)[:layers]) and splits(i)[layers:] == [33] * layers
+        assert all(n <= 4 for n in splits(i)[:layers]) and splits(i)[layers:] == [many] * layers
     # both decode: one launch, split by the longer context
-    assert calls(9, "qvl_attn_mfma_block") == [] and len(splits(9)) == layers and all(n >= 29 for n in splits(9))
+    assert calls(9, "qvl_attn_mfma_block") == [] and len(splits(9)) == layers and all(n == many for n in splits(9))
 
