@@ -10,8 +10,9 @@ out again to whoever asks next.
 
 Beside the pages every live request holds one *slot*, an index below ``max_num_seqs``.  A
 mixer with state of fixed size keeps it in row ``slot`` of its state tensor; the runner
-clears the row when the slot is taken.  The slot is also where the scheduler keeps the
-request's rope delta and sampler state.
+clears the row when the slot is taken.  Row ``slot`` of :class:`SlotRecords` (``records``) is the
+request's fixed-size record: its cached length, its rope delta and its sampler's state, filled at
+admission and gathered by slot index when a step is built and sampled.
 
 All of this is host bookkeeping; the tensors live in :class:`KVStorage`.
 """
@@ -24,6 +25,7 @@ from typing import Dict, List, Optional, Sequence, Tuple
 from ..parts.base import CacheNeed
 from .pages import OutOfPages, PagePool
 from .prefix import RadixPrefixCache
+from .slots import SlotRecords
 
 __all__ = ["CacheGroupSpec", "CacheManager", "RequestPages", "OutOfPages", "OutOfSlots"]
 
@@ -57,6 +59,7 @@ class CacheManager:
         self.max_num_seqs = int(max_num_seqs)
         self.pools = [PagePool(num_pages) for _ in self.groups]
         self._free_slots = list(range(self.max_num_seqs - 1, -1, -1))
+        self.records = SlotRecords(self.max_num_seqs)
         self.requests: Dict[object, RequestPages] = {}
         # A shared prefix is only valid where every group still holds all of its pages.
         self.prefix_cache: Optional[RadixPrefixCache] = None
@@ -64,13 +67,17 @@ class CacheManager:
             self.prefix_cache = RadixPrefixCache(self.pools, self.page_size, max_prefix_nodes)
 
     # ------------------------------------------------------------------ requests and slots
-    def admit(self, req_id) -> int:
+    def admit(self, req_id, params=None, rope_delta: int = 0, generated: int = 0) -> int:
+        """Give the request a slot and fill the slot's record: ``params`` are its sampling settings
+        (None: it is not sampled), ``rope_delta`` the offset of its text positions, ``generated`` the
+        tokens it has generated already (a request admitted again after it gave way)."""
         if req_id in self.requests:
             raise ValueError(f"request {req_id!r} is already live")
         if not self._free_slots:
             raise OutOfSlots(f"all {self.max_num_seqs} request slots are taken")
         slot = self._free_slots.pop()
         self.requests[req_id] = RequestPages(slot=slot, tables=[[] for _ in self.groups])
+        self.records.assign(slot, params, rope_delta, generated)
         return slot
 
     def slot_of(self, req_id) -> int:
@@ -92,6 +99,7 @@ class CacheManager:
             self.pools[g].free([p for p in table if p >= 0])
         if rp.prefix_nodes and self.prefix_cache is not None:
             self.prefix_cache.release(rp.prefix_nodes)
+        self.records.clear(rp.slot)
         self._free_slots.append(rp.slot)
 
     # ------------------------------------------------------------------ pages
@@ -135,6 +143,7 @@ class CacheManager:
         if num_tokens < rp.num_tokens:
             raise ValueError("a request's cached length cannot shrink")
         rp.num_tokens = num_tokens
+        self.records.num_tokens[rp.slot] = num_tokens
         for g, table in enumerate(rp.tables):
             first = min(self._first_needed_page(g, num_tokens), len(table))
             gone = [p for p in table[:first] if p >= 0]
@@ -177,6 +186,7 @@ class CacheManager:
                     raise OutOfPages("no page free for the copy of the page being filled")
         self.admit(dst_id)
         dst = self.requests[dst_id]
+        self.records.copy(src.slot, dst.slot)
         copies: List[Tuple[int, int, int]] = []
         for g, table in enumerate(src.tables):
             shared = list(table[:full])
@@ -207,6 +217,7 @@ class CacheManager:
             rp.tables[g] = list(pages[g])
         rp.prefix_nodes = nodes
         rp.num_tokens = matched
+        self.records.num_tokens[rp.slot] = matched
         return matched
 
     def register_prefix(self, req_id, tokens: Sequence[int], extra_keys: Optional[Sequence] = None) -> int:

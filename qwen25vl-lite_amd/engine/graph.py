@@ -118,10 +118,14 @@ class _Graph:
         cache, ps, h = self.parts.cache, self.ps, self.h
         n, b = len(entries), self.batch
         self.copied.synchronize()          # the previous transfer has read the pinned buffer
+        # where each request stands and the offset of its positions come from its slot's record,
+        # gathered by slot index
+        records = cache.records
+        at = np.fromiter((cache.requests[e.req_id].slot for e in entries), np.int64, n)
         starts = np.zeros(b, np.int32)     # rows from n on are padding: position 0, one key, no slot
         deltas = np.zeros(b, np.int32)
-        starts[:n] = np.fromiter((e.start for e in entries), np.int32, n)
-        deltas[:n] = np.fromiter((e.rope_delta for e in entries), np.int32, n)
+        starts[:n] = records.num_tokens[at]
+        deltas[:n] = records.rope_delta[at]
         tokens = h("token_ids")
         tokens[:n] = np.fromiter((e.tokens[0] for e in entries), np.int32, n)
         tokens[n:] = 0
@@ -129,7 +133,7 @@ class _Graph:
         h("positions", (self.rows, b))[:] = starts + deltas
         h("ctx_len")[:] = starts + 1
         slots_of = h("req_slots")
-        slots_of[:n] = np.fromiter((cache.slot_of(e.req_id) for e in entries), np.int32, n)
+        slots_of[:n] = at
         slots_of[n:] = self.parts.pad_state_slot
         for g in range(self.ngroups):
             table_np, lens, slots = self.tables[g], self.row_len[g], h(f"slots{g}")

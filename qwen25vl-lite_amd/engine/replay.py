@@ -61,6 +61,7 @@ class Replayer:
                 self.rope_delta[rid] = 0
             if "rope_delta" in e:
                 self.rope_delta[rid] = int(e["rope_delta"])
+                cache.records.rope_delta[cache.slot_of(rid)] = self.rope_delta[rid]
             entries.append(StepEntry(req_id=rid, tokens=list(e["tokens"]), start=cache.num_tokens(rid),
                                      want=list(e.get("want", [])), positions=e.get("positions"),
                                      rope_delta=self.rope_delta[rid]))

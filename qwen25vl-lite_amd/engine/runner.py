@@ -71,8 +71,8 @@ class ModelRunner:
             self.graphs.close()
 
     # ------------------------------------------------------------------ requests
-    def admit(self, req_id) -> int:
-        return self.cache.admit(req_id)
+    def admit(self, req_id, params=None, rope_delta: int = 0) -> int:
+        return self.cache.admit(req_id, params, rope_delta)
 
     def release(self, req_id) -> None:
         self.cache.release(req_id)
@@ -116,6 +116,9 @@ class ModelRunner:
                         raise ValueError(f"request {e.req_id!r}: token id outside [0, {self.vocab_size})")
                     if self.cache.num_tokens(e.req_id) != e.start:
                         raise ValueError(f"request {e.req_id!r}: the step does not continue where the cache ends")
+                    if self.cache.records.rope_delta[self.cache.slot_of(e.req_id)] != e.rope_delta:
+                        raise ValueError(f"request {e.req_id!r}: the entry's rope delta is not the one in its slot's "
+                                         "record (set at admission)")
                 logits = self.graphs.run(entries, device_tokens)
             elif device_tokens is not None:
                 raise ValueError("token ids on the device are taken by decode steps that run from a graph only")
@@ -138,6 +141,15 @@ class ModelRunner:
         from ..sampling.sampler import sample_rows_begin
         with torch.cuda.device(self.device):
             return sample_rows_begin(logits, params, prev_ids, steps)
+
+    def sample_slots_begin(self, logits: torch.Tensor, slots: Sequence[int], prev_ids: Sequence[Sequence[int]]):
+        """Queue the sampling of one token per logits row for the requests in ``slots``, whose
+        settings and sampler state lie in the cache manager's slot records; ``prev_ids`` are the
+        tokens each has generated (read for rows with penalties only).  Returns what
+        :meth:`sample_begin` returns."""
+        from ..sampling.sampler import sample_slots_begin
+        with torch.cuda.device(self.device):
+            return sample_slots_begin(logits, self.cache.records, slots, prev_ids)
 
     def sample(self, logits: torch.Tensor, params: Sequence, prev_ids: Sequence[Sequence[int]],
                steps: Sequence[int]) -> List[int]:

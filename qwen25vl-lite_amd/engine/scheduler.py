@@ -80,6 +80,7 @@ class Sequence_:
     cached_tokens: int = 0
     prompt_positions: Optional[List[List[int]]] = None   # [rows][prompt length], None = text
     rope_delta: int = 0
+    slot: int = -1                                       # its slot while it is running (see cache.SlotRecords)
     prefix_keys: Optional[List] = None
     arrival: float = field(default_factory=time.time)
     first_token_at: Optional[float] = None
@@ -169,6 +170,7 @@ class LLMEngine:
     def _preempt(self, victim: Sequence_) -> None:
         self.running.remove(victim)
         self.runner.cache.release(victim.seq_id)
+        victim.slot = -1
         victim.num_computed_tokens = 0
         victim.cached_tokens = 0
         victim.status = "waiting"
@@ -227,7 +229,8 @@ class LLMEngine:
             n = self._portion(seq, budget)
             if n <= 0:
                 break
-            cache.admit(seq.seq_id)
+            # the slot's record: sampling settings, rope delta, tokens generated before a preemption
+            seq.slot = cache.admit(seq.seq_id, seq.params, seq.rope_delta, len(seq.output_token_ids))
             adopted = 0
             if self.ecfg.enable_prefix_cache:
                 adopted = cache.adopt_prefix(seq.seq_id, seq.tokens, seq.prefix_keys)
@@ -236,6 +239,7 @@ class LLMEngine:
                 cache.reserve(seq.seq_id, adopted + n)
             except OutOfPages:
                 cache.release(seq.seq_id)
+                seq.slot = -1
                 if not self.running:
                     raise OutOfPages(f"request {seq.seq_id} cannot get pages for its first {adopted + n} tokens "
                                      "although nothing else is running") from None
@@ -305,13 +309,20 @@ class LLMEngine:
             if entry.want:
                 sampled.append(seq)
         if sampled:
-            args = ([s.params for s in sampled], [s.output_token_ids for s in sampled],
-                    [len(s.output_token_ids) for s in sampled])
             if ahead is not None and len(rows) < len(plan):
                 logits = logits[rows]          # every entry of a step queued ahead wants one row
+            prev = [s.output_token_ids for s in sampled]
+            by_slot = hasattr(self.runner, "sample_slots_begin")   # settings and sampler state from the slot records
+            if by_slot:
+                pending = self.runner.sample_slots_begin(logits, [s.slot for s in sampled], prev)
+            else:
+                args = ([s.params for s in sampled], prev, [len(p) for p in prev])
             if self._may_look_ahead(plan, sampled):
-                pending = self.runner.sample_begin(logits, *args)
+                if not by_slot:
+                    pending = self.runner.sample_begin(logits, *args)
                 self._queue_ahead(sampled, pending)
+                tokens = pending.result()
+            elif by_slot:
                 tokens = pending.result()
             else:
                 tokens = self.runner.sample(logits, *args)
@@ -364,6 +375,7 @@ class LLMEngine:
         """Append a sampled token and finish the request if it must (reference engine.py:831-872)."""
         params = seq.params
         seq.output_token_ids.append(token)
+        self.runner.cache.records.generated[seq.slot] += 1     # the sampler's state moves on with the token
         if seq.first_token_at is None:
             seq.first_token_at = time.time()
         reason: Optional[str] = None
@@ -380,6 +392,7 @@ class LLMEngine:
             return
         seq.status = "finished"
         self.runner.cache.release(seq.seq_id)
+        seq.slot = -1
         self.running.remove(seq)
         now = time.time()
         done.append(RequestOutput(

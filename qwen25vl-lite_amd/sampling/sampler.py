@@ -17,22 +17,27 @@ import torch
 from ..ops.kernels import KernelError, _check, _fn, _stream
 from .params import SamplingParams
 
-__all__ = ["sample_rows", "sample_rows_begin", "PendingSample", "uniform_for"]
+__all__ = ["sample_rows", "sample_rows_begin", "sample_slots_begin", "PendingSample", "uniform_for", "uniform_from"]
 
 _ROW = np.dtype([("temperature", "<f4"), ("top_p", "<f4"), ("min_p", "<f4"), ("u", "<f4"),
                  ("repetition", "<f4"), ("presence", "<f4"), ("frequency", "<f4"), ("top_k", "<i4"),
                  ("prev_begin", "<i4"), ("prev_end", "<i4")])
 
 
-def uniform_for(params: SamplingParams, step: int) -> float:
-    """The uniform number in [0, 1) for a request's output token number ``step``."""
-    if params.temperature <= 0:
-        return 0.0
-    if params.seed is None:
+def uniform_from(seed: Optional[int], step: int) -> float:
+    """The uniform number in [0, 1) for output token number ``step`` of a request with this seed
+    (None: from the global generator): a generator seeded with ``seed + step`` draws it
+    (the rule of reference engine.py:823-829)."""
+    if seed is None:
         return float(torch.rand(1).item())
     gen = torch.Generator()
-    gen.manual_seed(int(params.seed) + int(step))
+    gen.manual_seed(int(seed) + int(step))
     return float(torch.rand(1, generator=gen).item())
+
+
+def uniform_for(params: SamplingParams, step: int) -> float:
+    """The uniform number in [0, 1) for a request's output token number ``step``."""
+    return 0.0 if params.temperature <= 0 else uniform_from(params.seed, step)
 
 
 class _Staging:
@@ -131,6 +136,50 @@ def sample_rows_begin(logits: torch.Tensor, params: Sequence[SamplingParams], pr
         u = uniforms[i] if uniforms is not None else uniform_for(p, steps[i])
         rows[i] = (p.temperature, p.top_p, p.min_p, u, p.repetition_penalty, p.presence_penalty,
                    p.frequency_penalty, p.top_k if p.top_k else -1, begin, len(flat))
+    need_scores = any(p.temperature > 0 or len(flat) for p in params)
+    plain = any(p.temperature <= 0 and p.repetition_penalty == 1.0 and p.presence_penalty == 0.0
+                and p.frequency_penalty == 0.0 for p in params)
+    return _launch(logits, rows, flat, need_scores, plain)
+
+
+def sample_slots_begin(logits: torch.Tensor, records, slots: Sequence[int], prev_ids: Sequence[Sequence[int]],
+                       uniforms: Optional[Sequence[float]] = None) -> Optional[PendingSample]:
+    """:func:`sample_rows_begin` for requests whose settings and sampler state lie in their slots
+    (``records``: :class:`~qwen25vl_lite_amd.cache.slots.SlotRecords`): row ``m`` of the logits belongs to the
+    request in slot ``slots[m]``.  The rows' settings are gathered by slot index; only rows with
+    penalties (their generated tokens, ``prev_ids[m]``) and rows that draw (one generator each, by
+    the seed rule) are visited one by one."""
+    if not logits.is_cuda:
+        raise KernelError("sampling has no CPU path: logits must be on the GPU")
+    if logits.dtype != torch.float32 or logits.dim() != 2 or not logits.is_contiguous():
+        raise KernelError("logits must be contiguous float32 [M, vocab]")
+    m = logits.shape[0]
+    at = np.asarray(slots, np.int64)
+    if at.shape != (m,) or len(prev_ids) != m:
+        raise ValueError("one slot and token list per logits row is needed")
+    if m == 0:
+        return None
+    rows = np.zeros(m, _ROW)
+    for name in ("temperature", "top_p", "min_p", "top_k", "repetition", "presence", "frequency"):
+        rows[name] = getattr(records, name)[at]
+    flat: List[int] = []
+    draws = rows["temperature"] > 0
+    penal = (rows["repetition"] != 1.0) | (rows["presence"] != 0.0) | (rows["frequency"] != 0.0)
+    for i in np.nonzero(penal)[0]:
+        rows["prev_begin"][i] = len(flat)
+        flat.extend(int(t) for t in prev_ids[i])
+        rows["prev_end"][i] = len(flat)
+    for i in np.nonzero(draws)[0]:
+        seed = int(records.seed[at[i]])
+        rows["u"][i] = uniforms[i] if uniforms is not None else uniform_from(None if seed < 0 else seed,
+                                                                             int(records.generated[at[i]]))
+    return _launch(logits, rows, flat, bool(draws.any() or flat), bool((~draws & ~penal).any()))
+
+
+def _launch(logits: torch.Tensor, rows: np.ndarray, flat: List[int], need_scores: bool, plain: bool) -> PendingSample:
+    """Send the rows' settings to the device and queue the sampler.  ``need_scores``: some row scales
+    or penalises its logits (into a copy); ``plain``: some row is a plain argmax."""
+    m, vocab = logits.shape
     fn = _fn("sample", "qvl_sample_rows",
              [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
               ctypes.c_int, ctypes.c_int, ctypes.c_void_p])
@@ -139,13 +188,11 @@ def sample_rows_begin(logits: torch.Tensor, params: Sequence[SamplingParams], pr
         packed = np.concatenate([rows.view(np.int32), np.asarray(flat or [0], np.int32)])
         buf = _Staging.to_device(packed, dev)
         n_row_words = rows.view(np.int32).size
-        need_scores = any(p.temperature > 0 or len(flat) for p in params)
         scores = torch.empty_like(logits) if need_scores else logits
         out = torch.empty(m, dtype=torch.int32, device=dev)
         # a greedy row without penalties is a plain argmax: several blocks scan it side by side
         parts = None
-        if any(p.temperature <= 0 and p.repetition_penalty == 1.0 and p.presence_penalty == 0.0
-               and p.frequency_penalty == 0.0 for p in params):
+        if plain:
             part_bytes = int(_fn("sample", "qvl_sample_argmax_part_bytes", [])())
             parts = torch.empty(m * part_bytes, dtype=torch.uint8, device=dev)
         _check(fn(logits.data_ptr(), scores.data_ptr(), buf.data_ptr(), buf[n_row_words:].data_ptr(),

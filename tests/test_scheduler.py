@@ -382,3 +382,39 @@ def test_finished_outputs_are_handed_over_once():
     eng.add_request([3, 4], SamplingParams(max_tokens=2, ignore_eos=True))
     outs = eng.run_until_complete()
     assert len(outs) == 1 and outs[0].prompt_token_ids == [3, 4]
+
+
+def test_the_slot_record_follows_its_request():
+    """Every live request's slot holds its fixed-size record: cached length, rope delta, sampler
+    settings and the number of tokens it has generated (what the seed rule draws from).  The record
+    is filled at admission, moves on with every step, survives a preemption (the request is admitted
+    again with what it had generated) and is cleared when the slot is given back."""
+    eng, runner = _engine(num_blocks=6, block_size=16, max_num_seqs=3, max_num_batched_tokens=64,
+                          enable_prefix_cache=False)
+    rec = runner.cache.records
+    a = eng.add_request(list(range(1, 31)), SamplingParams(temperature=0.7, top_k=5, seed=11, max_tokens=40, ignore_eos=True))
+    b = eng.add_request(list(range(2, 22)), SamplingParams(max_tokens=40, repetition_penalty=1.3, ignore_eos=True),
+                        rope_delta=4)
+    seqs = {s.seq_id: s for s in eng.waiting}
+    preempted = False
+    for _ in range(400):
+        eng.step()
+        preempted = preempted or eng.stats_.preemptions > 0
+        for s in eng.running:
+            slot = runner.cache.slot_of(s.seq_id)
+            assert s.slot == slot
+            assert rec.num_tokens[slot] == s.num_computed_tokens == runner.cache.num_tokens(s.seq_id)
+            assert rec.generated[slot] == len(s.output_token_ids)
+            assert rec.rope_delta[slot] == s.rope_delta
+            assert rec.seed[slot] == (-1 if s.params.seed is None else s.params.seed)
+            assert rec.temperature[slot] == pytest.approx(s.params.temperature) and rec.top_k[slot] == s.params.top_k
+            assert rec.repetition[slot] == pytest.approx(s.params.repetition_penalty)
+        free = set(range(3)) - {runner.cache.slot_of(s.seq_id) for s in eng.running}
+        for slot in free:      # a slot nobody holds has the record of a plain greedy request
+            assert rec.num_tokens[slot] == rec.generated[slot] == rec.rope_delta[slot] == 0 and rec.seed[slot] == -1
+            assert rec.temperature[slot] == 0 and rec.repetition[slot] == 1 and rec.top_k[slot] == -1
+        if not eng.has_work():
+            break
+    assert preempted, "the pool is small enough that one of the two had to give way and come back"
+    assert seqs[a].status == seqs[b].status == "finished" and not eng.has_work()
+    assert rec.plain_greedy(__import__("numpy").arange(3))
