@@ -153,36 +153,24 @@ def measure_peaks(torch):
     read_l2 = _fn("peaks", "qvl_peak_read_again", [c_ptr, c_ll, c_int, c_ptr, c_int, c_ptr])
     ms = best_ms(lambda: _check(read_l2(small.data_ptr(), small.numel() // 16, reps, flag.data_ptr(), cus * 8, _stream()), "read"))
     out["read_2MiB_by_every_block_from_L2_TBps"] = round(cus * 8 * small.numel() * reps / ms / 1e9, 3)
+    # v_mfma_f32_16x16x32_bf16 back to back on registers, eight independent chains a wave.  Blocks of
+    # 1,024 threads (four waves on every SIMD, which stay there together), two such blocks a compute
+    # unit: the rate, the clock the shader really ran at (its own cycle counter against the constant
+    # 100 MHz clock, read around one wave's loop) and the cycles between two of a wave's instructions.
+    # A slow clock would show in the second figure, an instruction that cannot be issued faster in the third.
     iters, blocks = 4096, cus * 8
-    ms = best_ms(lambda: _check(mfma(flag.data_ptr(), iters, blocks, 256, None, _stream()), "mfma"))
-    flops = blocks * 4 * iters * 8 * 2.0 * 16 * 16 * 32
-    out["mfma_16x16x32_bf16_PFLOPs"] = round(flops / ms / 1e12, 3)
-    # The same loop with the shader's cycle counter and the constant 100 MHz clock read around it, with
-    # one, two and four waves on every SIMD, first as that many blocks of four waves a compute unit
-    # (which the dispatcher does not keep resident side by side all the time), then as one block of
-    # that many waves a SIMD for every compute unit (which it must).  A slow clock would show in the
-    # clock, an instruction that cannot be issued faster in the cycles a SIMD spends per
-    # instruction while the waves of one block take turns on it.
     clocks = torch.zeros(2 * blocks, dtype=torch.int64, device="cuda")
-    for label, threads, per_cu in (("1_wave_a_simd", 256, 1), ("2_waves_a_simd_two_blocks", 256, 2),
-                                   ("4_waves_a_simd_four_blocks", 256, 4), ("8_waves_a_simd_eight_blocks", 256, 8),
-                                   ("2_waves_a_simd_one_block", 512, 1), ("4_waves_a_simd_one_block", 1024, 1),
-                                   ("8_waves_a_simd_two_blocks_of_16", 1024, 2)):
+    for label, threads, per_cu in (("", 1024, 2), ("_one_block_of_8_waves_a_cu", 512, 1), ("_blocks_of_4_waves", 256, 8)):
         n = cus * per_cu
         launch = lambda: _check(mfma(flag.data_ptr(), iters, n, threads, clocks.data_ptr(), _stream()), "mfma")
         for _ in range(3):      # the clock settles under load
             launch()
-        ms = best_ms(launch, reps=3)
-        torch.cuda.synchronize()
+        ms = best_ms(launch, reps=5)
         c = clocks.view(blocks, 2)[:n].double()
         cycles, wall_s = c[:, 0].median().item(), c[:, 1].median().item() / 100e6
-        together = threads // 256    # waves of one block on a SIMD
-        out[f"mfma_{label}"] = {
-            "shader_clock_GHz": round(cycles / wall_s / 1e9, 3),
-            "cycles_per_instruction_of_a_wave": round(cycles / (iters * 8), 2),
-            "cycles_per_instruction_of_the_block_per_simd": round(cycles / (together * iters * 8), 2),
-            "loop_ms": round(wall_s * 1e3, 3), "kernel_ms": round(ms, 3),
-            "PFLOPs": round(n * (threads // 64) * iters * 8 * 2.0 * 16 * 16 * 32 / ms / 1e12, 3)}
+        out[f"mfma_16x16x32_bf16{label}_PFLOPs"] = round(n * (threads // 64) * iters * 8 * 2.0 * 16 * 16 * 32 / ms / 1e12, 3)
+        out[f"mfma_16x16x32_bf16{label}_shader_clock_GHz"] = round(cycles / wall_s / 1e9, 3)
+        out[f"mfma_16x16x32_bf16{label}_cycles_between_a_waves_instructions"] = round(cycles / (iters * 8), 2)
     # an empty kernel many times in a row, from the host and from a graph
     n = 200
     ms = best_ms(lambda: _check(empty(n, _stream()), "empty"))
