@@ -16,7 +16,7 @@ LIBRARIES = [
     ("gemm_f32", {}),
     ("sample", {}),
     ("gemm_resident", {}),
-    ("gemm_chunked", {}),
+    ("gemm_split", {}),
     ("peaks", {}),
     # the matrix-core attention is compiled per head size; these are the sizes the tests and the
     # benchmark use, any other multiple of 16 is compiled at its first use

@@ -77,11 +77,11 @@ def linear_into(residual: Optional[torch.Tensor], x: torch.Tensor, weight: torch
     """``residual += x @ weight.T`` inside the product's kernel where that exists (few bfloat16
     rows): then None is returned.  Otherwise what is to be added is returned and the caller hands
     it on to whoever adds it (the next norm's kernel): the product ``[M, N]``, or float32
-    ``[slabs, M, N]`` whose slabs are added in order (the chunked kernel)."""
+    ``[slabs, M, N]`` whose slabs are added in order (the split kernel)."""
     m, k = x.shape
     fast = x.is_cuda and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and _aligned(x)
-    if fast and skinny.prefers_chunked(m, k, weight):
-        return skinny.chunked_product(weight, x)
+    if fast and skinny.prefers_split(m, k, weight):
+        return skinny.split_product(weight, x)
     if (fast and m <= skinny.ONE_BLOCK_ROWS and residual is not None and skinny.takes_resident(m, k, weight)
             and residual.dtype == torch.float32 and residual.shape == (m, weight.shape[0]) and residual.stride(1) == 1):
         skinny.resident_product(weight, x=x, epilogue=skinny.RESIDUAL, out=residual)

@@ -15,10 +15,11 @@ import torch
 
 from .kernels import _check, _fn, _ptr, _stream, dtype_code
 
-__all__ = ["resident_product", "takes_resident", "qkv_rope_product", "takes_qkv_rope", "RESIDENT_ROWS", "resident_norm_k", "resident_two_tile_k", "folds_norm", "TEAM_LONG_K", "ONE_BLOCK_ROWS", "chunked_product", "takes_chunked", "prefers_chunked", "CHUNKED_ROWS",
+__all__ = ["resident_product", "takes_resident", "qkv_rope_product", "takes_qkv_rope", "RESIDENT_ROWS", "resident_norm_k", "resident_two_tile_k", "folds_norm", "TEAM_LONG_K", "ONE_BLOCK_ROWS", "split_product", "takes_split", "prefers_split", "SPLIT_ROWS",
            "STORE", "RESIDUAL", "SWIGLU"]
 
 RESIDENT_ROWS = 64       # up to here the resident kernel runs
+ONE_TILE_ROWS = 16       # the rows of one column tile of the matrix instruction
 ONE_BLOCK_ROWS = 32      # up to here one block carries all rows: beyond, teams of blocks share the weight's
                          # tiles, which pays for the fused q | k | v projection only
 TEAM_LONG_K = 1          # flag: 17 to 32 rows with a long inner size go to a team of two blocks
@@ -181,44 +182,52 @@ def qkv_rope_product(weight: torch.Tensor, cs: torch.Tensor, *, x: Optional[torc
     return q_out
 
 
-CHUNKED_ROWS = (17, 64)   # the rows the chunked kernel is built for
+SPLIT_ROWS = 64   # the most rows the split kernel is built for
 
 
-def takes_chunked(m: int, k: int, weight: torch.Tensor) -> bool:
-    """Whether the chunked kernel (``csrc/gemm_chunked.hip``) takes a product of ``m`` rows with this
-    weight: 17 to 64 bfloat16 rows, whose partial sums over chunks of the inner size come back as
+def takes_split(m: int, k: int, weight: torch.Tensor) -> bool:
+    """Whether the split kernel (``csrc/gemm_split.hip``) takes a product of ``m`` rows with this
+    weight: up to 64 bfloat16 rows, whose partial sums over chunks of the inner size come back as
     slabs."""
-    return (CHUNKED_ROWS[0] <= m <= CHUNKED_ROWS[1] and k % 8 == 0 and weight.dtype == torch.bfloat16
-            and _rows_aligned(weight, 8))
-
-
-def prefers_chunked(m: int, k: int, weight: torch.Tensor) -> bool:
-    """Where the chunked kernel is the fastest of the three (measured on MI355X at the 7B decoder's
-    shapes): 17 to 32 rows with an inner size too long for the rows to stay in one block (the down
-    projection: 38 us against the resident kernel's 58), and 33 to 64 rows against a matrix so
-    small that the library's tiles do not fill the device (the output projection)."""
-    if not takes_chunked(m, k, weight):
+    if not (1 <= m <= SPLIT_ROWS and k % 8 == 0 and weight.dtype == torch.bfloat16 and _rows_aligned(weight, 8)):
         return False
-    if m <= ONE_BLOCK_ROWS:
-        return k > resident_two_tile_k()
-    return weight.shape[0] * k <= (1 << 24)
+    n = weight.shape[0]
+    if ((n - 1) * weight.stride(0) + k) * 2 >= _MAX_WEIGHT_BYTES:
+        return False
+    cus = _compute_units(weight.device)
+    return int(_fn("gemm_split", "qvl_gemm_split_chunks", [_c_int, _c_int, _c_int, _c_int])(m, n, k, cus)) > 0
 
 
-def chunked_product(weight: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
+def prefers_split(m: int, k: int, weight: torch.Tensor) -> bool:
+    """Where the split kernel is the fastest way to a product that is added to the residual
+    (measured on MI355X at the 3B, 7B and 72B decoders' output and down projections): up to 16 rows
+    when the inner size is too long for a block of the resident kernel to keep its rows for one
+    pass over the weight (the down projection at 8 rows: 26.9 us against 37.3, which pays for the
+    norm kernel that then adds the slabs, 5.7 us, where the resident kernel adds in place and the
+    next product forms the norm itself); with more rows always (the output projection at 32 rows:
+    9.9 us and a norm kernel of 6 against 14.3 in place and 8 more for the norm inside the gate | up
+    product; at 64 rows 14.4 us against the library's 13.9 to 17.6, the down projection 36.2
+    against 46.6)."""
+    if not takes_split(m, k, weight):
+        return False
+    return m > ONE_TILE_ROWS or k > resident_norm_k()
+
+
+def split_product(weight: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
     """Partial sums of ``x @ weight.T`` over chunks of the inner size: float32 ``[chunks, M, N]``,
     whose sum over the first axis (taken in order by whoever reads them: the norm that follows) is
     the product.  ``x`` is bfloat16 ``[M, K]``."""
     m = x.shape[0]
     n, k = weight.shape
-    if not takes_chunked(m, k, weight) or x.shape[1] != k:
-        raise ValueError("the chunked kernel does not take this product")
+    if not takes_split(m, k, weight) or x.shape[1] != k:
+        raise ValueError("the split kernel does not take this product")
     if x.dtype != torch.bfloat16 or not _rows_aligned(x, 8):
         raise ValueError("x must be bfloat16 with 16-byte aligned rows")
     cus = _compute_units(x.device)
-    chunks = int(_fn("gemm_chunked", "qvl_gemm_chunked_chunks", [_c_int, _c_int, _c_int])(n, k, cus))
+    chunks = int(_fn("gemm_split", "qvl_gemm_split_chunks", [_c_int, _c_int, _c_int, _c_int])(m, n, k, cus))
     out = torch.empty((chunks, m, n), dtype=torch.float32, device=x.device)
-    fn = _fn("gemm_chunked", "qvl_gemm_chunked",
+    fn = _fn("gemm_split", "qvl_gemm_split",
              [_c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr])
     _check(fn(_ptr(x), x.stride(0), _ptr(weight), weight.stride(0), _ptr(out), m, n, k, cus, _stream()),
-           "linear (chunked)")
+           "linear (split)")
     return out

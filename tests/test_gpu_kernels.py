@@ -423,9 +423,9 @@ def test_product_added_into_the_residual(m, n, k):
     h = torch.randn(m, n).cuda()
     want = h.cpu() + x.float().cpu() @ w.float().cpu().T
     left = linear_into(h, x, w)
-    if m <= 16 or (m <= 32 and k <= 3840):      # one block carries the rows: added in place
+    if m <= 16 and k <= 4096:      # one block carries the rows for the whole inner size: added in place
         assert left is None and torch.allclose(h.cpu(), want, atol=3e-3, rtol=3e-3)
-    elif m <= 32 or (m <= 64 and n * k <= 1 << 24):   # the chunked kernel: slabs of partial sums for the next norm to add
+    elif m <= 64:   # the split kernel: slabs of partial sums for the next norm to add
         assert left.dtype == torch.float32 and left.dim() == 3 and tuple(left.shape[1:]) == (m, n)
         assert torch.allclose(h.cpu() + left.sum(0).cpu(), want, atol=3e-3, rtol=3e-3)
     else:   # the library's product comes back in bfloat16 for the next norm to add
@@ -457,22 +457,28 @@ def test_gate_up_product_with_the_activation_folded_in(dtype, m, inter, k):
 
 
 @pytest.mark.parametrize("m, n, k", [(64, 3584, 18944), (17, 509, 352), (33, 130, 200), (48, 1000, 3584), (40, 144, 352),
-                                     (64, 37, 8), (25, 4700, 1248), (57, 300, 1256)])
-def test_chunked_product_and_the_norm_that_adds_its_slabs(m, n, k):
-    """17 to 64 rows against a weight cut along its inner size: the slabs of partial sums add up to
-    the product (inner sizes that are no multiple of 32, row counts that fill no tile), twice the
-    same bits; and the norm kernel that takes the slabs as its addend gives what it gives for
-    their sum."""
+                                     (64, 37, 8), (25, 4700, 1248), (57, 300, 1256), (1, 3584, 18944), (8, 2048, 11008),
+                                     (16, 37, 4104), (3, 5000, 2056), (49, 8, 2048 * 300 + 8)])
+def test_split_product_and_the_norm_that_adds_its_slabs(m, n, k):
+    """Up to 64 rows against a weight cut along its inner size: the slabs of partial sums add up to
+    the product (inner sizes that are no multiple of 32, row counts that fill no tile, more chunks
+    than compute units refused), twice the same bits; and the norm kernel that takes the slabs as
+    its addend gives what it gives for their sum."""
     from qwen25vl_lite_amd.ops import kernels, skinny
     torch.manual_seed(n + k)
     w = (torch.randn(n, k) / math.sqrt(k)).bfloat16()
     x = torch.randn(m, k).bfloat16()
     want = x.float() @ w.float().T
-    assert skinny.takes_chunked(m, k, w.cuda()) and not skinny.takes_chunked(16, k, w.cuda())
-    slabs = skinny.chunked_product(w.cuda(), x.cuda())
+    if k > 2048 * 256:
+        assert not skinny.takes_split(m, k, w.cuda())
+        with pytest.raises(ValueError):
+            skinny.split_product(w.cuda(), x.cuda())
+        return
+    assert skinny.takes_split(m, k, w.cuda()) and not skinny.takes_split(65, k, w.cuda())
+    slabs = skinny.split_product(w.cuda(), x.cuda())
     assert slabs.dtype == torch.float32 and slabs.dim() == 3 and tuple(slabs.shape[1:]) == (m, n)
     assert torch.allclose(slabs.sum(0).cpu(), want, atol=3e-3, rtol=3e-3), (slabs.sum(0).cpu() - want).abs().max()
-    assert torch.equal(slabs, skinny.chunked_product(w.cuda(), x.cuda()))
+    assert torch.equal(slabs, skinny.split_product(w.cuda(), x.cuda()))
     if n % 4 == 0:
         h = torch.randn(m, n).cuda()
         g = (1 + 0.1 * torch.randn(n)).cuda()
