@@ -133,7 +133,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
 
 // The addend as slabs of partial sums (float32 [slab][row][H], H a multiple of 4 and at most
 // SLAB_VEC_MAX * 4096): a block of 1024 threads per row, a thread per 4 neighbouring values, the
-// slabs' loads asked for eight at a time (they do not depend on each other, only the sum has an
+// slabs' loads asked for sixteen at a time (they do not depend on each other, only the sum has an
 // order: slab 0, 1, 2, ...).
 #define SLAB_VEC_MAX 2
 template <typename TO>
@@ -147,24 +147,27 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_slabs_kernel(float* __restri
   float* hr = h + (size_t)row * H;
   const float* dr = delta + (size_t)row * H;
   const int nvec = H >> 2;
-  float4 v[SLAB_VEC_MAX];
+  float4 v[SLAB_VEC_MAX], g[SLAB_VEC_MAX];
   float ss = 0.f;
 #pragma unroll
   for (int j = 0; j < SLAB_VEC_MAX; ++j) {
     const int i = threadIdx.x + 1024 * j;
     if (i < nvec) {
+      // everything the thread needs is asked for before anything is waited for: the row of h, the
+      // norm's weights and up to 16 slabs
+      float4 x = ld4<float>(hr + 4 * i);
+      g[j] = ld4<float>(w + 4 * i);
       float4 d = {0.f, 0.f, 0.f, 0.f};
-      for (int c0 = 0; c0 < nslabs; c0 += 8) {
-        float4 e[8];
+      for (int c0 = 0; c0 < nslabs; c0 += 16) {
+        float4 e[16];
 #pragma unroll
-        for (int c = 0; c < 8; ++c)
+        for (int c = 0; c < 16; ++c)
           e[c] = c0 + c < nslabs ? ld4<float>(dr + (size_t)(c0 + c) * slab_stride + 4 * i) : float4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int c = 0; c < 8; ++c) {
+        for (int c = 0; c < 16; ++c) {
           if (c0 + c < nslabs) { d.x += e[c].x; d.y += e[c].y; d.z += e[c].z; d.w += e[c].w; }
         }
       }
-      float4 x = ld4<float>(hr + 4 * i);
       x.x += d.x; x.y += d.y; x.z += d.z; x.w += d.w;
       if (!rows) st4<float>(hr + 4 * i, x);
       v[j] = x;
@@ -176,10 +179,8 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_slabs_kernel(float* __restri
 #pragma unroll
   for (int j = 0; j < SLAB_VEC_MAX; ++j) {
     const int i = threadIdx.x + 1024 * j;
-    if (i < nvec) {
-      const float4 g = ld4<float>(w + 4 * i);
-      st4<TO>(o + 4 * i, float4{(v[j].x * rs) * g.x, (v[j].y * rs) * g.y, (v[j].z * rs) * g.z, (v[j].w * rs) * g.w});
-    }
+    if (i < nvec)
+      st4<TO>(o + 4 * i, float4{(v[j].x * rs) * g[j].x, (v[j].y * rs) * g[j].y, (v[j].z * rs) * g[j].z, (v[j].w * rs) * g[j].w});
   }
 }
 
