@@ -512,13 +512,13 @@ struct Plan {
   int mt, groups;
   bool one_pass;
 };
-static Plan plan_for(int M, int K, bool norm, int blocks, bool prefer_teams) {
+static Plan plan_for(int M, int K, bool norm, int blocks) {
   if (M <= 16) return Plan{1, 1, K <= PASS_K};
   const bool two_fit = K <= 32 * XHI_STEPS;
   if (M <= 32 && two_fit) return Plan{2, 1, true};
   if (two_fit && blocks >= 8 * ((M + 31) / 32)) return Plan{2, (M + 31) / 32, true};
   const int singles = (M + 15) / 16;
-  if ((M > 32 || prefer_teams || norm) && blocks >= 8 * singles) return Plan{1, singles, K <= PASS_K};
+  if ((M > 32 || norm) && blocks >= 8 * singles) return Plan{1, singles, K <= PASS_K};
   if (M <= 32) return Plan{2, 1, false};
   return Plan{0, 1, false};
 }
@@ -549,7 +549,7 @@ static int launch(ResidentArgs p, const Plan& pl, int blocks, hipStream_t stream
 // many compute units.
 extern "C" int qvl_gemm_resident_folds_norm(int M, int K, int blocks) {
   if (M <= 0 || M > 64 || K <= 0 || K > PASS_K || blocks <= 0) return 0;
-  const Plan pl = plan_for(M, K, true, blocks, false);
+  const Plan pl = plan_for(M, K, true, blocks);
   return pl.one_pass && pl.mt <= 2;
 }
 
@@ -573,16 +573,14 @@ extern "C" int qvl_gemm_resident_two_tile_k() { return 32 * XHI_STEPS; }
 // max_blocks: blocks to launch at most (the number of compute units).
 extern "C" int qvl_gemm_resident(const void* x, int ldx, const void* h, int ldh, const void* norm_w, float eps,
                                  const void* W, int ldw, const void* bias, void* out, int ldo, int M, int N, int K,
-                                 int out_dtype, int epilogue, int max_blocks, int flags, hipStream_t stream) {
-  // flags bit 0: 17 to 32 rows with a long K go to a team of two blocks rather than to one block
-  // that reads its rows again for every pass
+                                 int out_dtype, int epilogue, int max_blocks, hipStream_t stream) {
   if (M <= 0 || N <= 0) return QVL_OK;
   if (M > 64) return QVL_ERR_LIMIT;
   if (M > 32 && K > PASS_K) return QVL_ERR_LIMIT;   // teams of more than two keep their rows for a single pass
   if (K <= 0 || K % 8 || ldw % 8 || ldw < K || max_blocks <= 0 || !W || !out) return QVL_ERR_SHAPE;
   if (!fits_descriptors(M, N, K, ldw, ldx, ldh, ldo)) return QVL_ERR_LIMIT;
   const bool norm = h != nullptr;
-  const Plan pl = plan_for(M, K, norm, max_blocks, flags & 1);
+  const Plan pl = plan_for(M, K, norm, max_blocks);
   const int teams = plan_teams(pl, max_blocks);
   if (norm) {
     if (x || !norm_w || K > PASS_K || ldh % 4 || ldh < K) return QVL_ERR_SHAPE;
@@ -652,7 +650,7 @@ extern "C" int qvl_gemm_resident_rope(const void* x, int ldx, const void* h, int
   if (nq <= 0 || nkv < 0 || hd <= 0 || hd % 16 || ps <= 0 || !cs) return QVL_ERR_SHAPE;
   if (nkv > 0 && (!slot || !kc || !vc)) return QVL_ERR_SHAPE;
   const bool norm = h != nullptr;
-  const Plan pl = plan_for(M, K, norm, max_blocks, false);
+  const Plan pl = plan_for(M, K, norm, max_blocks);
   const int teams = plan_teams(pl, max_blocks);
   if (norm) {
     if (x || !norm_w || K > PASS_K || ldh % 4 || ldh < K) return QVL_ERR_SHAPE;

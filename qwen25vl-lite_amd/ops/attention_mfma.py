@@ -19,15 +19,35 @@ __all__ = ["try_attention", "supports", "tiles_for", "plan_splits"]
 
 _c_int, _c_float, _c_ptr = ctypes.c_int, ctypes.c_float, ctypes.c_void_p
 _MAX_HD = 256
-TARGET_BLOCKS = 512        # from here on a wave per tile fills the 256 compute units
-FILL_BLOCKS = 256          # with fewer cooperative blocks than this, contexts are split among blocks
+# Thresholds that follow the device: counts per compute unit (measured on 256 of them); the names below
+# them hold a number instead of None where a caller (a test) fixes the count itself.
+TARGET_PER_CU = 2          # from this many (tile, head) pairs a compute unit on, a wave per tile fills the device
+FILL_PER_CU = 1            # with fewer cooperative blocks than this, contexts are split among blocks
+WIDE_WALKS_PER_CU = 3      # the kind of the kernel whose waves carry three column tiles: from this many walks on
+WIDE_BLOCKS_PER_CU = 586   # ... that have this many 32-key blocks to walk between them (150,000 on 256 units)
+TARGET_BLOCKS = None
+FILL_BLOCKS = None
 MIN_KEYS_PER_SPLIT = 1024  # merging the splits (stores, a counter and loads that go through to memory) costs a decode
                            # step about as much as each wave's walk over four more 32-key blocks: shorter splits lose
 MERGE_COUNTERS = 1 << 16   # (tile, kv head) pairs whose splits one launch can merge by itself
 ALONE_KEYS = 4096          # decoded tokens beside prompt portions get a launch of their own from this context on
-WIDE_WALKS = 768           # the kind of the kernel whose waves carry three column tiles: from this many walks on
-WIDE_BLOCKS = 150_000      # ... that have this many 32-key blocks to walk between them
 WIDE_CT = 3
+_cu_count = {}
+
+
+def _compute_units(device=None) -> int:
+    key = torch.device(device).index if device is not None and torch.device(device).index is not None else torch.cuda.current_device()
+    if key not in _cu_count:
+        _cu_count[key] = torch.cuda.get_device_properties(key).multi_processor_count
+    return _cu_count[key]
+
+
+def _target_blocks(device=None) -> int:
+    return TARGET_BLOCKS if TARGET_BLOCKS is not None else TARGET_PER_CU * _compute_units(device)
+
+
+def _fill_blocks(device=None) -> int:
+    return FILL_BLOCKS if FILL_BLOCKS is not None else FILL_PER_CU * _compute_units(device)
 
 
 def supports(head_dim: int, dtype: torch.dtype) -> bool:
@@ -68,14 +88,14 @@ def tiles_for(cu_q, group: int, tile_ct: int = 1, ctx_len=None) -> Tuple[np.ndar
     return req, ct
 
 
-def plan_splits(num_tiles: int, nkv: int, max_ctx: int) -> Tuple[str, int, int]:
+def plan_splits(num_tiles: int, nkv: int, max_ctx: int, device=None) -> Tuple[str, int, int]:
     """``(kernel, nsplit, keys_per_split)``.  ``"tile"``: many tiles, as in prefill: a block owns
     several tiles per wave and shares the keys through LDS.  ``"coop"``: the waves of a block share a tile (few tiles, as in decode); its keys are
     split among ``nsplit`` blocks when the context is long and the blocks are few."""
     blocks = num_tiles * nkv
-    if blocks >= TARGET_BLOCKS:
+    if blocks >= _target_blocks(device):
         return "tile", 1, 0
-    want = (FILL_BLOCKS + blocks - 1) // blocks
+    want = (_fill_blocks(device) + blocks - 1) // blocks
     nsplit = max(1, min(want, max_ctx // MIN_KEYS_PER_SPLIT))
     if nsplit == 1:
         return "coop", 1, 0
@@ -134,7 +154,7 @@ def _walk_blocks(step, group: int, tile_ct: int, only=None) -> int:
     return int((entries * np.maximum(1, (ctx - q // 2 + 31) // 32)).sum())
 
 
-def long_single_tiles(step, group: int, nkv: int):
+def long_single_tiles(step, group: int, nkv: int, device=None):
     """In a step that has prompt portions too: the requests whose tokens make one tile only
     (decoded tokens) if they are few and their contexts long, as a tuple of 0/1 per request, else
     None.  Planned together with the portions, each of them gets one workgroup (or one block) that
@@ -147,7 +167,7 @@ def long_single_tiles(step, group: int, nkv: int):
     if not single.any() or single.all():
         return None
     longest = int(np.asarray(step.ctx_len_host, dtype=np.int64)[single].max())
-    if longest < ALONE_KEYS or int(single.sum()) * nkv >= FILL_BLOCKS:
+    if longest < ALONE_KEYS or int(single.sum()) * nkv >= _fill_blocks(device):
         return None
     return tuple(int(x) for x in single)
 
@@ -181,13 +201,15 @@ def try_attention(q, k_cache, v_cache, block_table, step, num_q_heads: int, wind
     tile_req, tile_ct, num_tiles = _step_tiles(step, nq // nkv, 1, q.device)
     out = torch.empty_like(q)
     defines = {"HD": hd}
-    kind, nsplit, per = plan_splits(num_tiles, nkv, step.max_ctx_len)
+    kind, nsplit, per = plan_splits(num_tiles, nkv, step.max_ctx_len, q.device)
 
     def many_tiles(only):
         tile_req, tile_ct, num_tiles = _step_tiles(step, nq // nkv, block_tiles(hd), q.device, by_length=True, only=only)
         wide = force_wide
         if wide is None:   # many and long walks: measured at the 7B decoder's heads, the wide kind wins from one prompt of about 8,192 tokens on
-            wide = hd <= 128 and num_tiles * nkv >= WIDE_WALKS and _walk_blocks(step, nq // nkv, block_tiles(hd), only) * nkv >= WIDE_BLOCKS
+            cus = _compute_units(q.device)
+            wide = (hd <= 128 and num_tiles * nkv >= WIDE_WALKS_PER_CU * cus
+                    and _walk_blocks(step, nq // nkv, block_tiles(hd), only) * nkv >= WIDE_BLOCKS_PER_CU * cus)
         defines = block_defines(hd, wide)
         if wide:
             tile_req, tile_ct, num_tiles = _step_tiles(step, nq // nkv, block_tiles(hd, True), q.device, by_length=True, only=only)
@@ -235,14 +257,14 @@ def try_attention(q, k_cache, v_cache, block_table, step, num_q_heads: int, wind
                   int(window or 0), float(scale), nsplit, per, _stream()),
                "paged_attention (matrix cores, shared tiles)")
 
-    single = long_single_tiles(step, nq // nkv, nkv) if force_groups is None else None
+    single = long_single_tiles(step, nq // nkv, nkv, q.device) if force_groups is None else None
     if single is not None:   # the few decoded tokens with long contexts by themselves, the rest planned anew
         longest = max(c for c, s in zip(step.ctx_len_host, single) if s)
-        _, nsplit1, per1 = plan_splits(sum(single), nkv, longest)   # fewer blocks than FILL_BLOCKS: the kernel that splits
+        _, nsplit1, per1 = plan_splits(sum(single), nkv, longest, q.device)   # fewer blocks than fill the device: the kernel that splits
         shared_tiles(single, nsplit1, per1)
         rest = tuple(1 - s for s in single)
         kind, nsplit, per = plan_splits(_step_tiles(step, nq // nkv, 1, q.device, only=rest)[2], nkv,
-                                        max(c for c, s in zip(step.ctx_len_host, rest) if s))
+                                        max(c for c, s in zip(step.ctx_len_host, rest) if s), q.device)
         if kind == "tile":
             many_tiles(rest)
         else:

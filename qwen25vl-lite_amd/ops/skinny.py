@@ -15,14 +15,13 @@ import torch
 
 from .kernels import _check, _fn, _ptr, _stream, dtype_code
 
-__all__ = ["resident_product", "takes_resident", "qkv_rope_product", "takes_qkv_rope", "RESIDENT_ROWS", "resident_norm_k", "resident_two_tile_k", "folds_norm", "TEAM_LONG_K", "ONE_BLOCK_ROWS", "split_product", "takes_split", "prefers_split", "SPLIT_ROWS",
+__all__ = ["resident_product", "takes_resident", "qkv_rope_product", "takes_qkv_rope", "RESIDENT_ROWS", "resident_norm_k", "resident_two_tile_k", "folds_norm", "ONE_BLOCK_ROWS", "split_product", "takes_split", "prefers_split", "SPLIT_ROWS",
            "STORE", "RESIDUAL", "SWIGLU"]
 
 RESIDENT_ROWS = 64       # up to here the resident kernel runs
 ONE_TILE_ROWS = 16       # the rows of one column tile of the matrix instruction
 ONE_BLOCK_ROWS = 32      # up to here one block carries all rows: beyond, teams of blocks share the weight's
                          # tiles, which pays for the fused q | k | v projection only
-TEAM_LONG_K = 1          # flag: 17 to 32 rows with a long inner size go to a team of two blocks
 _MAX_WEIGHT_BYTES = 0xffffff00   # qvl_gemm_resident_max_weight_bytes() + 1
 _pass_k = None
 _two_tile_k = None
@@ -92,8 +91,7 @@ def takes_resident(m: int, k: int, weight: torch.Tensor, *, norm: bool = False) 
 def resident_product(weight: torch.Tensor, *, x: Optional[torch.Tensor] = None, h: Optional[torch.Tensor] = None,
                      norm_weight: Optional[torch.Tensor] = None, eps: float = 0.0,
                      bias: Optional[torch.Tensor] = None, epilogue: int = STORE,
-                     out: Optional[torch.Tensor] = None, out_dtype: torch.dtype = torch.float32,
-                     flags: int = 0) -> torch.Tensor:
+                     out: Optional[torch.Tensor] = None, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
     """``X @ weight.T`` for at most 64 rows (``h`` for at most 32).  ``X`` is ``x`` (bfloat16), or ``rmsnorm(h) * norm_weight``
     formed inside the kernel from the float32 rows ``h``.  ``epilogue``: ``STORE`` writes the product
     (plus ``bias``) to a new tensor of ``out_dtype``; ``RESIDUAL`` adds it to ``out`` (float32) in
@@ -123,10 +121,10 @@ def resident_product(weight: torch.Tensor, *, x: Optional[torch.Tensor] = None, 
         out, odt = torch.empty((m, n), dtype=out_dtype, device=src.device), out_dtype
     fn = _fn("gemm_resident", "qvl_gemm_resident",
              [_c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_float, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int,
-              _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+              _c_int, _c_int, _c_int, _c_int, _c_ptr])
     _check(fn(_ptr(x), x.stride(0) if x is not None else 0, _ptr(h), h.stride(0) if h is not None else 0,
               _ptr(norm_weight), float(eps), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(out), out.stride(0),
-              m, n, k, dtype_code(odt), epilogue, _compute_units(src.device), int(flags), _stream()),
+              m, n, k, dtype_code(odt), epilogue, _compute_units(src.device), _stream()),
            "linear (resident)")
     return out
 

@@ -201,7 +201,7 @@ def test_paged_attention_matrix_cores(nq, nkv, hd, window, ps, split, monkeypatc
     groups = {"tile": 1, "tile_two_groups": 2}.get(split)
     if groups == 2 and hd > 128:
         pytest.skip("two groups of waves are built for head sizes up to 128")
-    monkeypatch.setattr(attention_mfma, "plan_splits", lambda t, n, m: plan)
+    monkeypatch.setattr(attention_mfma, "plan_splits", lambda t, n, m, d=None: plan)
     cu = [0]
     for ql in c["qlens"]:
         cu.append(cu[-1] + ql)
@@ -280,13 +280,13 @@ def test_paged_attention_long_portions(nq, nkv, hd, window, ps):
                        max_ctx_len=max(lens), dtype=torch.bfloat16)
     import unittest.mock as mock
     for groups in (1, 2) if hd <= 128 else (1,):   # an odd and an even number of key blocks among the walks
-        with mock.patch.object(attention_mfma, "plan_splits", lambda t, n, m: ("tile", 1, 0)):
+        with mock.patch.object(attention_mfma, "plan_splits", lambda t, n, m, d=None: ("tile", 1, 0)):
             out = attention_mfma.try_attention(c["q"], c["kc"], c["vc"], c["table"], step, nq, window, c["scale"],
                                                force_groups=groups, force_wide=False)
         err = (out.float().cpu() - c["want"]).abs().max()
         assert torch.allclose(out.float().cpu(), c["want"], atol=1.5e-2, rtol=2e-2), (groups, err)
     if hd in (128, 48):   # the kind whose waves carry three column tiles (its operands pass through a few registers)
-        with mock.patch.object(attention_mfma, "plan_splits", lambda t, n, m: ("tile", 1, 0)):
+        with mock.patch.object(attention_mfma, "plan_splits", lambda t, n, m, d=None: ("tile", 1, 0)):
             out = attention_mfma.try_attention(c["q"], c["kc"], c["vc"], c["table"], step, nq, window, c["scale"],
                                                force_groups=1, force_wide=True)
         err = (out.float().cpu() - c["want"]).abs().max()
@@ -297,7 +297,7 @@ def test_paged_attention_long_portions(nq, nkv, hd, window, ps):
     assert int(attention_mfma._work_queue(c["q"].device)[0].abs().sum()) == 0
     assert attention_mfma.block_groups(10, 512, hd) == (2 if hd <= 128 else 1)
     assert attention_mfma.block_groups(513, 512, hd) == 1
-    with mock.patch.object(attention_mfma, "plan_splits", lambda t, n, m: ("tile", 1, 0)), pytest.raises(kernels.KernelError):
+    with mock.patch.object(attention_mfma, "plan_splits", lambda t, n, m, d=None: ("tile", 1, 0)), pytest.raises(kernels.KernelError):
         attention_mfma.try_attention(c["q"], c["kc"], c["vc"], c["table"], step, nq, window, c["scale"], force_groups=3)
 
 
@@ -362,23 +362,6 @@ def test_linear_bfloat16(m, n, k):
     if m > 1:
         alone = linear(x[m // 2:m // 2 + 1].contiguous().cuda(), w.cuda(), out_dtype=torch.float32)
         assert torch.allclose(alone[0], out32[m // 2], atol=1e-5, rtol=1e-5)
-
-
-@pytest.mark.parametrize("m, n, k", [(17, 300, 8200), (32, 3584, 18944), (25, 130, 4104)])
-def test_team_of_two_blocks_for_a_long_inner_size(m, n, k):
-    """17 to 32 rows whose inner size does not fit one pass: on request two blocks of one XCD walk
-    the same tiles, each with 16 of the rows (the kernel's other way is one block that reads its rows
-    again for every pass); both give the product."""
-    from qwen25vl_lite_amd.ops import skinny
-    torch.manual_seed(m)
-    x, w = torch.randn(m, k).bfloat16().cuda(), (torch.randn(n, k) / math.sqrt(k)).bfloat16().cuda()
-    want = x.float() @ w.float().T
-    team = skinny.resident_product(w, x=x, out_dtype=torch.float32, flags=skinny.TEAM_LONG_K)
-    assert torch.allclose(team, want, atol=2e-3, rtol=2e-3)
-    res = torch.randn(m, n).cuda()
-    into = res.clone()
-    skinny.resident_product(w, x=x, epilogue=skinny.RESIDUAL, out=into, flags=skinny.TEAM_LONG_K)
-    assert torch.allclose(into, res + want, atol=2e-3, rtol=2e-3)
 
 
 @pytest.mark.parametrize("m, n, k", [(1, 48, 64), (7, 1000, 3584), (16, 130, 4096), (3, 64, 144),
