@@ -324,7 +324,9 @@ def main(argv=None) -> int:
             torch.cuda.synchronize()
             return time.perf_counter() - t0, outs, engine.stats()
 
+        from qwen25vl_lite_amd.ops import attention_mfma
         serve()                                   # library tuning, kernel builds, graph captures
+        attention_mfma.taken.clear()
         sec, outs, stats = serve()
         generated = sum(len(o.output_token_ids) for o in outs)
         prompt_tokens = sum(len(tk) for tk, _ in reqs)
@@ -335,7 +337,8 @@ def main(argv=None) -> int:
             "generated_tokens": generated, "prompt_tokens": prompt_tokens, "steps": int(stats["steps"]),
             "prefix_cache_hits": int(stats["prefix_cache_hits"]),
             "prefix_cache_tokens_saved": int(stats["prefix_cache_tokens_saved"]),
-            "preemptions": int(stats["preemptions"]), "data": "synthetic"}))
+            "preemptions": int(stats["preemptions"]), "data": "synthetic",
+            "attention_kernels": dict(attention_mfma.taken)}))
         return 0
     if args.prefill_only:
         sec = prefill_rate(2048)
@@ -344,8 +347,12 @@ def main(argv=None) -> int:
     # The prefill is measured first: of the workloads here it is the one bound by the matrix cores,
     # whose clocks give way once the device has been kept busy for a while (after the decode runs of
     # this program's default length the same prefill takes a few per cent longer).
+    from qwen25vl_lite_amd.ops import attention_mfma
     prefill_sec = None if args.no_points else prefill_rate(2048)
+    kinds = {"prefill_2048": dict(attention_mfma.taken)}
+    attention_mfma.taken.clear()
     value, ms_per_step, ctx_mid = decode_rate(args.batch, args.steps, args.warmup)
+    kinds["prompts_and_decode"] = dict(attention_mfma.taken)   # launches by kind; a captured decode step counts once
     need = step_bytes(t, args.batch, ctx_mid, 2 if args.dtype == "bfloat16" else 4)
     achieved = need / (ms_per_step * 1e-3) / 1e9
     peak_key = "bf16" if args.dtype == "bfloat16" else "fp32"
@@ -377,6 +384,7 @@ def main(argv=None) -> int:
         flops = prefill_flops(t, tokens)
         line["prefill"] = {"value": round(tokens / sec, 1), "tokens": tokens, "ms": round(sec * 1e3, 3),
                            "frac": round(flops / sec / MFMA_PEAK[peak_key], 4)}
+    line["attention_kernels"] = kinds
     print(json.dumps(line))
     return 0
 

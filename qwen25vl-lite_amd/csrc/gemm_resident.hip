@@ -8,7 +8,9 @@
 // rows of W (= outputs); the host picks `rows` so that the tiles divide evenly among the compute
 // units (3584 outputs on 256 units: 256 tiles of 14 rather than 224 of 16), the matrix-core tile's
 // other rows stay zero.
-// Wave w covers the 256 values of K from 256 w on, as the A operand (W rows) and B operand (X
+// Wave w covers the 32 RK values of K from 32 RK w on (RK = 8: 256; a second build with RK = 4 serves
+// inner sizes up to 2,048, where with 256 values a wave half the waves would have none and the
+// other half would carry all loads), as the A operand (W rows) and B operand (X
 // rows) of v_mfma_f32_16x16x32_bf16; the 16 waves' sums meet in LDS and are added in wave order.
 // Up to 16 rows of X are one column tile of the matrix instruction; 17 to 32 rows are two (MT = 2):
 // every W fragment that is loaded is multiplied with both.  More rows are spread over teams of
@@ -81,7 +83,9 @@ extern "C" void qvl_gemm_resident_timeline(void* p) { timeline_buffer = (unsigne
 #define W_RING 2   // half-step buffers of W that go round
 #endif
 #define RW 16   // waves per block
-#define RK 8    // 32-wide K steps per wave and pass
+#ifndef RK
+#define RK 8    // 32-wide K steps per wave and pass (the host loads a build with 4 for inner sizes up to 2,048: all 16 waves then have columns)
+#endif
 #define PASS_K (RW * RK * 32)
 #define XHI_STEPS 120   // 32-wide K steps of the second column tile that fit LDS beside the sums: K <= 3840
 
@@ -192,7 +196,8 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
       // hold whole rows between them.  Loads return in the order they are issued: the rows and
       // the norm weights are asked for first and W (by first_w) right behind them, so the
       // statistics and the scaling run while W is still on its way.  A lane fetches 4 of its
-      // wave's 256 norm weights; they reach the lanes that need them through LDS.
+      // wave's 32 RK norm weights (the first 8 RK lanes do); they reach the lanes that need them
+      // through LDS.
       const uint32_t at = m_ok ? ((uint32_t)row * p.ldh + k_lane) * 4 : PAST_END;
       const int inside = steps_inside(0);
       float4 v[RK][2];
@@ -203,8 +208,10 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
         v[u][1] = __builtin_bit_cast(float4, buffer_load16(h_buf, o, u * 128 + 16));
       }
       const int kg = wave * RK * 32 + 4 * lane;
+      const bool gain_lane = 4 * lane < RK * 32;
       // beyond K the descriptor's own size gives zeros (K is a multiple of 8, kg of 4)
-      const float4 g4 = __builtin_bit_cast(float4, buffer_load16(gain_buf, again ? PAST_END : (uint32_t)kg * 4));
+      const float4 g4 =
+          __builtin_bit_cast(float4, buffer_load16(gain_buf, (again || !gain_lane) ? PAST_END : (uint32_t)kg * 4));
       first_w();
       float ss = 0.f;
 #pragma unroll
@@ -217,7 +224,7 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
       STAMP(6);   // this wave's rows have arrived
       if (again) __syncthreads();   // the other column tile's statistics have been read
       if (lg == 0) rowsq[wave][r] = ss;
-      if (!again) *reinterpret_cast<float4*>(&gains[wave][4 * lane]) = g4;
+      if (!again && gain_lane) *reinterpret_cast<float4*>(&gains[wave][4 * lane]) = g4;
       __syncthreads();
       STAMP(7);   // every wave's have
       float total = 0.f;

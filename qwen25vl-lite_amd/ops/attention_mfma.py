@@ -7,6 +7,7 @@ tile list depends on the batch and on the group size only and is built once per 
 
 from __future__ import annotations
 
+import collections
 import ctypes
 from typing import Optional, Tuple
 
@@ -106,6 +107,7 @@ def plan_splits(num_tiles: int, nkv: int, max_ctx: int, device=None) -> Tuple[st
 
 _queues = {}
 _merge_counters = {}
+taken = collections.Counter()   # launches by kind of kernel (a captured launch counts once): what a measurement reports
 
 
 def _counters(device: torch.device) -> torch.Tensor:
@@ -228,6 +230,7 @@ def try_attention(q, k_cache, v_cache, block_table, step, num_q_heads: int, wind
             # whatever a launch that went wrong did to the counters, the next one starts from zero
             queue.zero_()
         _check(code, "paged_attention (matrix cores)")
+        taken[f"many tiles, {WIDE_CT if wide else 2} column tiles a wave, {groups} wave group{'s' if groups > 1 else ''}"] += 1
 
     def shared_tiles(only, nsplit, per):
         tile_req, tile_ct, num_tiles = _step_tiles(step, nq // nkv, 1, q.device, only=only)
@@ -248,6 +251,7 @@ def try_attention(q, k_cache, v_cache, block_table, step, num_q_heads: int, wind
             if code:
                 counters.zero_()
             _check(code, "paged_attention (matrix cores, shared tiles, merged)")
+            taken["shared tiles, keys split among blocks, merged in the launch"] += 1
             return
         fn = _fn("attention_mfma", "qvl_attn_mfma_coop",
                  [_c_ptr] * 4 + [_c_int] + [_c_ptr] * 4 + [_c_int, _c_ptr, _c_ptr] + [_c_int] * 4
@@ -256,6 +260,7 @@ def try_attention(q, k_cache, v_cache, block_table, step, num_q_heads: int, wind
                   _ptr(step.ctx_len), _ptr(tile_req), _ptr(tile_ct), num_tiles, _ptr(out), _ptr(scratch), nq, nkv, ps,
                   int(window or 0), float(scale), nsplit, per, _stream()),
                "paged_attention (matrix cores, shared tiles)")
+        taken["shared tiles" + (", keys split among blocks, merged by a second launch" if nsplit > 1 else "")] += 1
 
     single = long_single_tiles(step, nq // nkv, nkv, q.device) if force_groups is None else None
     if single is not None:   # the few decoded tokens with long contexts by themselves, the rest planned anew

@@ -16,6 +16,7 @@ LIBRARIES = [
     ("gemm_f32", {}),
     ("sample", {}),
     ("gemm_resident", {}),
+    ("gemm_resident", {"RK": 4}),
     ("gemm_split", {}),
     ("peaks", {}),
     # the matrix-core attention is compiled per head size; these are the sizes the tests and the
