@@ -91,6 +91,8 @@ def takes_resident(m: int, k: int, weight: torch.Tensor, *, norm: bool = False) 
         return False     # the kernel reaches its operands through 32-bit byte offsets
     if norm:
         return folds_norm(m, k, weight.device)
+    if k <= NARROW_K:
+        return True      # one pass in either build, with any number of rows (and no question to the other build)
     if m > 32:
         return k <= resident_norm_k()    # teams keep their rows for one pass; in several passes they lose to the library
     if k <= (resident_norm_k() if m <= 16 else resident_two_tile_k()):
@@ -218,7 +220,7 @@ def prefers_split(m: int, k: int, weight: torch.Tensor) -> bool:
     against 46.6)."""
     if not takes_split(m, k, weight):
         return False
-    return m > ONE_TILE_ROWS or k > resident_norm_k()
+    return m > ONE_TILE_ROWS or (k > NARROW_K and k > resident_norm_k())
 
 
 def split_product(weight: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
