@@ -480,6 +480,34 @@ def test_split_product_and_the_norm_that_adds_its_slabs(m, n, k):
         assert torch.equal(h3, h) and torch.allclose(c3, kernels.add_rmsnorm(h.clone(), total, g, 1e-6, torch.float32)[[m - 1, 0]])
 
 
+def test_few_row_products_at_random_sizes():
+    """The resident kernel (both builds: inner sizes up to and beyond 2,048) and the split kernel at
+    sizes drawn at random: any row count up to 64, widths that fill no tile, inner sizes in steps of 8
+    on either side of a pass, of a chunk and of a build; every one against the float32 product."""
+    import random
+    from qwen25vl_lite_amd.ops import skinny
+    from qwen25vl_lite_amd.ops.linear import linear, linear_into
+    rng = random.Random(5)
+    edges = [8, 120, 128, 136, 1016, 1024, 2040, 2048, 2056, 3832, 3840, 3848, 4088, 4096, 4104, 6144, 8200]
+    for case in range(48):
+        m = rng.choice([1, 2, 7, 15, 16, 17, 31, 32, 33, 47, 48, 49, 63, 64])
+        n = rng.choice([1, 5, 15, 16, 17, 100, 255, 256, 257, 1000])
+        k = rng.choice(edges) if case % 2 else 8 * rng.randint(1, 700)
+        torch.manual_seed(case)
+        x = torch.randn(m, k).bfloat16().cuda()
+        w = (torch.randn(n, k) / math.sqrt(k)).bfloat16().cuda()
+        want = x.float() @ w.float().T
+        got = linear(x, w, out_dtype=torch.float32)
+        assert torch.allclose(got, want, atol=5e-3, rtol=5e-3), (m, n, k, (got - want).abs().max().item())
+        slabs = skinny.split_product(w, x)
+        assert torch.allclose(slabs.sum(0), want, atol=5e-3, rtol=5e-3), (m, n, k, (slabs.sum(0) - want).abs().max().item())
+        h = torch.randn(m, n).cuda()
+        before = h.clone()
+        left = linear_into(h, x, w)
+        total = h if left is None else h + (left.sum(0) if left.dim() == 3 else left.float())
+        assert torch.allclose(total, before + want, atol=2e-2, rtol=2e-2), (m, n, k)
+
+
 def test_no_cpu_path():
     from qwen25vl_lite_amd.ops import kernels
     from qwen25vl_lite_amd.ops.linear import linear
