@@ -79,9 +79,7 @@ extern "C" void qvl_gemm_resident_timeline(void* p) { timeline_buffer = (unsigne
 #define STAMP(i)
 #endif
 
-#ifndef W_RING
 #define W_RING 2   // half-step buffers of W that go round
-#endif
 #define RW 16   // waves per block
 #ifndef RK
 #define RK 8    // 32-wide K steps per wave and pass (the host loads a build with 4 for inner sizes up to 2,048: all 16 waves then have columns)
@@ -407,10 +405,9 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
 
   if (ONE_PASS || MT == 1) {
     // The block's work is a sequence of steps: every tile of its own, and within a tile every pass
-    // over K (one, if X stays resident).  Three half-step buffers of W go round: while a step is
-    // multiplied, the first half of the next is on its way; its second half and the first half of
-    // the step after it are asked for as soon as the product has freed their registers, and arrive
-    // during the merge of the sums (or, between the passes of a tile, while the next rows of X come).
+    // over K (one, if X stays resident).  Two half-step buffers of W go round: each is asked for
+    // again, for the next step, as soon as the product has freed its registers, and arrives during
+    // the merge of the sums (or, between the passes of a tile, while the next rows of X come).
     const int passes = ONE_PASS ? 1 : (p.K + PASS_K - 1) / PASS_K;
     auto step_after = [&](int& t, int& ps) {
       if (++ps >= passes) {
@@ -439,26 +436,18 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
     }
     STAMP(1);   // the rows are in their registers, the first tile asked for
     Epi e = epi_load(tile);
-#if W_RING == 3
-    {
-      int t1 = tile, p1 = 0;
-      step_after(t1, p1);
-      load_w_part(t1, p1 * PASS_K, 0, RK / 2, w[2]);
-    }
-#endif
     Acc acc = zero;
     // one step whose halves are in a_lo and a_hi; false: it was the block's last
     // A half buffer is asked for again the moment its steps are multiplied (not after the whole
     // step).  Between the passes of a tile the next rows of X are asked for the same way, each half
     // ahead of the W half that is needed with it (loads come back in the order they were asked
     // for).  Every step issues the same loads, a step beyond the block's last one past the end of
-    // the buffers.  With a ring of three half buffers the half that is free takes the first half of
-    // the step after next; with two, each half takes its own part of the next step.
+    // the buffers.  (A ring of three half buffers, the free one taking the first half of the step
+    // after next, needs more registers than a lane has: the compiler spills, and a spill's scratch
+    // store makes every wait a wait for everything.)
     auto one = [&](bf16x8_t* a_lo, bf16x8_t* a_hi) {
       int tn = tile, pn = pass;
       step_after(tn, pn);
-      int ta = tn, pa = pn;
-      step_after(ta, pa);
       const bool tile_done = ONE_PASS || pn == 0;
       // the order below is the order of the instructions: the compiler's scheduler would pull the
       // loads of later steps ahead of the products and run out of registers for them
@@ -467,14 +456,13 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
       if (tile == team) { asm volatile("s_nop 0" :: "v"(acc.t[0])); STAMP(2); }   // the first half tile was there
       HOLD_ORDER();
       if (!ONE_PASS && MT == 1) load_x_half(pn * PASS_K, 0, xb);
-      load_w_part(tn, pn * PASS_K, W_RING == 3 ? RK / 2 : 0, RK / 2, a_lo);
+      load_w_part(tn, pn * PASS_K, 0, RK / 2, a_lo);
       HOLD_ORDER();
       acc = product_part(a_hi, RK / 2, RK / 2, xb, nullptr, acc);
       HOLD_ORDER();
       const Epi e_next = epi_load(tn);
       if (!ONE_PASS && MT == 1) load_x_half(pn * PASS_K, 1, xb);
-      if (W_RING == 3) load_w_part(ta, pa * PASS_K, 0, RK / 2, a_hi);
-      else load_w_part(tn, pn * PASS_K, RK / 2, RK / 2, a_hi);
+      load_w_part(tn, pn * PASS_K, RK / 2, RK / 2, a_hi);
       HOLD_ORDER();
       if (tile_done) {
         if (tile == team) STAMP(3);   // all of the first tile multiplied
@@ -489,10 +477,6 @@ __global__ __launch_bounds__(64 * RW) void gemm_resident_kernel(ResidentArgs p) 
     };
     while (tile < p.ntiles) {
       if (!one(w[0], w[1])) break;
-#if W_RING == 3
-      if (!one(w[2], w[0])) break;
-      if (!one(w[1], w[2])) break;
-#endif
     }
     STAMP(5);
   } else {
