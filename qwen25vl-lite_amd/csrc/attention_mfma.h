@@ -18,7 +18,9 @@ long long qvl_attn_mfma_scratch_floats(int num_tiles, int nkv, int nsplit);
 // Attention of few column tiles (decode): the waves of a block share a tile; with nsplit > 1 the
 // keys of a tile are cut into nsplit ranges of keys_per_split keys (a multiple of 32) whose partial
 // results go through `scratch` (qvl_attn_mfma_scratch_floats() floats, the caller's) and are
-// merged by a second kernel.
+// merged by a second kernel.  tile_req and tile_ct may both be null: tile i is then the one tile of
+// request i; cu_q may be null: every request then brings one token, request r the token r (a step
+// of decoded tokens only: the kernel starts without reading either).
 int qvl_attn_mfma_coop(const void* q, const void* kc, const void* vc, const void* bt, int table_width,
                        const void* cu_q, const void* ctx_len, const void* tile_req, const void* tile_ct,
                        int num_tiles, void* out, void* scratch, int nq, int nkv, int ps, int window, float scale,

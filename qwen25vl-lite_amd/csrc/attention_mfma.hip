@@ -404,10 +404,22 @@ struct TileInfo {
   int lo_tile, hi_tile;
 };
 
+// A request's run of tokens in this step.  Without the array of run starts every request brings one
+// token, request r the token r (a step of decoded tokens only): nothing is read then.
+struct Run {
+  int q0, qlen;
+};
+__device__ __forceinline__ Run run_of(const int* cu_q, int r) {
+  if (!cu_q) return Run{r, 1};
+  const int q0 = cu_q[r];
+  return Run{q0, cu_q[r + 1] - q0};
+}
+
 __device__ __forceinline__ TileInfo tile_info(const int* cu_q, const int* ctx_len, int r, int ct, int g, int kvh,
                                               int window) {
   const int lane = threadIdx.x & 63, c = lane & 15;
-  const int q0 = cu_q[r], qlen = cu_q[r + 1] - q0, ctx = ctx_len[r];
+  const Run run = run_of(cu_q, r);
+  const int q0 = run.q0, qlen = run.qlen, ctx = ctx_len[r];
   const int col = ct * 16 + c;
   const int i = col / g, gh = col - i * g;
   TileInfo t;
@@ -876,7 +888,8 @@ __device__ __forceinline__ float load_device_scope(const float* p) {
 template <bool ACROSS>
 __device__ __forceinline__ void merge_splits(const float* __restrict__ base, int nsplit, int r, int ct, int kvh, int g,
                                              const int* __restrict__ cu_q, bf16_t* __restrict__ out, int nq) {
-  const int q0 = cu_q[r], qlen = cu_q[r + 1] - q0;
+  const Run run = run_of(cu_q, r);
+  const int q0 = run.q0, qlen = run.qlen;
   for (int idx = threadIdx.x; idx < 16 * (HD / 4); idx += blockDim.x) {
     const int col = idx / (HD / 4), d = (idx - col * (HD / 4)) * 4;
     const int colg = ct * 16 + col;
@@ -933,7 +946,8 @@ __global__ __launch_bounds__(64 * COOP_WAVES) void attn_mfma_coop_kernel(
   const int tile = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lg = lane >> 4, c = lane & 15;
   const int g = nq / nkv;
-  const int r = tile_req[tile], ct = tile_ct[tile];
+  // without a tile list tile i is the only tile of request i
+  const int r = tile_req ? tile_req[tile] : tile, ct = tile_req ? tile_ct[tile] : 0;
   const TileInfo t = tile_info(cu_q, ctx_len, r, ct, g, kvh, window);
   int first = t.lo_tile, last = t.hi_tile;
   if (nsplit > 1) {  // splits are cut by absolute key index, in multiples of 32
@@ -980,7 +994,8 @@ __global__ __launch_bounds__(64 * COOP_WAVES) void attn_mfma_coop_kernel(
     }
     const int colg = ct * 16 + col;
     const int i = colg / g, gh = colg - i * g;
-    const int q0 = cu_q[r], qlen = cu_q[r + 1] - q0;
+    const Run run = run_of(cu_q, r);
+    const int q0 = run.q0, qlen = run.qlen;
     if (nsplit > 1) {
       float* part = scratch + (((size_t)tile * nkv + kvh) * nsplit + split) * PART_STRIDE + (size_t)col * PART_COLS;
       if (counters) {   // read by another block of this launch
@@ -1026,8 +1041,8 @@ __global__ void attn_mfma_merge_kernel(const float* __restrict__ scratch, const 
                                        bf16_t* __restrict__ out, int nq, int nkv, int nsplit) {
   // one block per (tile, kv head)
   const int tile = blockIdx.x, kvh = blockIdx.y;
-  merge_splits<false>(scratch + ((size_t)tile * nkv + kvh) * nsplit * PART_STRIDE, nsplit, tile_req[tile], tile_ct[tile],
-                      kvh, nq / nkv, cu_q, out, nq);
+  merge_splits<false>(scratch + ((size_t)tile * nkv + kvh) * nsplit * PART_STRIDE, nsplit, tile_req ? tile_req[tile] : tile,
+                      tile_req ? tile_ct[tile] : 0, kvh, nq / nkv, cu_q, out, nq);
 }
 
 static int check_common(int num_tiles, int nq, int nkv, int ps, int table_width) {

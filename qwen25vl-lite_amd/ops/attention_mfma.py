@@ -234,6 +234,11 @@ def try_attention(q, k_cache, v_cache, block_table, step, num_q_heads: int, wind
 
     def shared_tiles(only, nsplit, per):
         tile_req, tile_ct, num_tiles = _step_tiles(step, nq // nkv, 1, q.device, only=only)
+        cu_q = step.cu_q
+        if only is None and step.max_q_len == 1 and num_tiles == step.num_reqs == len(step.cu_q_host) - 1 == step.cu_q_host[-1]:
+            # decoded tokens only: request i brings token i and has tile i, and the kernel is told so
+            # instead of reading it (two dependent reads less before its first key is asked for)
+            tile_req = tile_ct = cu_q = None
         scratch = None
         if nsplit > 1:
             floats = _fn("attention_mfma", "qvl_attn_mfma_scratch_floats", [_c_int] * 3, defines)
@@ -245,7 +250,7 @@ def try_attention(q, k_cache, v_cache, block_table, step, num_q_heads: int, wind
             fn = _fn("attention_mfma", "qvl_attn_mfma_coop_merged",
                      [_c_ptr] * 4 + [_c_int] + [_c_ptr] * 4 + [_c_int, _c_ptr, _c_ptr, _c_ptr] + [_c_int] * 4
                      + [_c_float, _c_int, _c_int, _c_ptr], defines)
-            code = fn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(step.cu_q),
+            code = fn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(cu_q),
                       _ptr(step.ctx_len), _ptr(tile_req), _ptr(tile_ct), num_tiles, _ptr(out), _ptr(scratch),
                       _ptr(counters), nq, nkv, ps, int(window or 0), float(scale), nsplit, per, _stream())
             if code:
@@ -256,7 +261,7 @@ def try_attention(q, k_cache, v_cache, block_table, step, num_q_heads: int, wind
         fn = _fn("attention_mfma", "qvl_attn_mfma_coop",
                  [_c_ptr] * 4 + [_c_int] + [_c_ptr] * 4 + [_c_int, _c_ptr, _c_ptr] + [_c_int] * 4
                  + [_c_float, _c_int, _c_int, _c_ptr], defines)
-        _check(fn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(step.cu_q),
+        _check(fn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(cu_q),
                   _ptr(step.ctx_len), _ptr(tile_req), _ptr(tile_ct), num_tiles, _ptr(out), _ptr(scratch), nq, nkv, ps,
                   int(window or 0), float(scale), nsplit, per, _stream()),
                "paged_attention (matrix cores, shared tiles)")

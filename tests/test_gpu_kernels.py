@@ -224,6 +224,46 @@ def test_paged_attention_matrix_cores(nq, nkv, hd, window, ps, split, monkeypatc
         assert int(attention_mfma._counters(c["q"].device).abs().sum()) == 0
 
 
+@pytest.mark.parametrize("split", ["coop", "coop_split", "coop_split_two_kernels"])
+@pytest.mark.parametrize("nq, nkv, hd, window", [(14, 2, 128, None), (6, 2, 48, 100), (8, 8, 16, 7)])
+def test_a_step_of_decoded_tokens_only(nq, nkv, hd, window, split, monkeypatch):
+    """Every request brings one token: the kernel is not handed the lists of tiles and of run
+    starts (tile i is request i's, its token is token i) and gives what it gives with them."""
+    from qwen25vl_lite_amd.ops import attention_mfma
+    from qwen25vl_lite_amd.parts import StepContext
+    lens = (333, 17, 64, 1, 200)
+    c = _attention_case(torch.bfloat16, nq, nkv, hd, window, lens, (1,) * len(lens))
+    plan = ("coop", 1, 0) if split == "coop" else ("coop", 6, 64)
+    if split == "coop_split_two_kernels":
+        monkeypatch.setattr(attention_mfma, "MERGE_COUNTERS", 0)
+    monkeypatch.setattr(attention_mfma, "plan_splits", lambda t, n, m, d=None: plan)
+    cu = list(range(len(lens) + 1))
+    none = torch.zeros(0, dtype=torch.int32).cuda()
+    step = StepContext(num_tokens=len(lens), num_reqs=len(lens), token_ids=none, positions=none, token_req=c["req"],
+                       token_seqpos=c["seqpos"], cu_q=torch.tensor(cu, dtype=torch.int32).cuda(),
+                       ctx_len=torch.tensor(lens, dtype=torch.int32).cuda(), req_slots=none, groups=[],
+                       logit_rows=none, cu_q_host=cu, ctx_len_host=list(lens), max_q_len=1, max_ctx_len=max(lens),
+                       dtype=torch.bfloat16)
+    handed = []
+    real = attention_mfma._fn
+
+    def spy(stem, name, *a, **k):
+        fn = real(stem, name, *a, **k)
+        if not name.startswith("qvl_attn_mfma_coop"):
+            return fn
+        return lambda *args: (handed.append((args[5], args[7], args[8])), fn(*args))[1]   # cu_q, tile_req, tile_ct
+
+    monkeypatch.setattr(attention_mfma, "_fn", spy)
+    out = attention_mfma.try_attention(c["q"], c["kc"], c["vc"], c["table"], step, nq, window, c["scale"])
+    assert handed == [(None, None, None)]
+    assert torch.allclose(out.float().cpu(), c["want"], atol=1.5e-2, rtol=2e-2), (out.float().cpu() - c["want"]).abs().max()
+    # the same step declared as one that might hold portions: the lists are handed over, the result is the same bits
+    step.max_q_len = 2
+    handed.clear()
+    with_lists = attention_mfma.try_attention(c["q"], c["kc"], c["vc"], c["table"], step, nq, window, c["scale"])
+    assert handed and handed[0][0] is not None and torch.equal(with_lists, out)
+
+
 @pytest.mark.parametrize("nq, nkv, hd, window", [(14, 2, 128, None), (6, 2, 48, 100)])
 def test_mixed_step_with_few_long_decoded_tokens(nq, nkv, hd, window, monkeypatch):
     """A prompt portion beside two decoded tokens whose contexts are long: the decoded tokens go to
