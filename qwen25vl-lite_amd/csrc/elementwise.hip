@@ -288,12 +288,22 @@ __global__ void rope_kv_write_kernel(const TI* __restrict__ x, int x_stride, con
 // The same for float32 sums, bfloat16 outputs and the table of cosines and sines in hand, with
 // all widths multiples of 4 (the prompt portions of a bfloat16 run): a block per token, a thread
 // per 4 neighbouring channels, 16-byte loads and 8-byte stores.
+// x may come as nslabs slabs, slab_stride elements apart (partial sums of a product cut along its inner
+// size): they are added in slab order, then the bias.
 __global__ __launch_bounds__(256) void rope_kv_write_wide_kernel(
     const float* __restrict__ x, int x_stride, const float* __restrict__ bias, const float2* __restrict__ cs,
     const int* __restrict__ slot, bf16_t* __restrict__ q_out, bf16_t* __restrict__ kc, bf16_t* __restrict__ vc, int nq,
-    int nkv, int hd, int rot_half, int ps) {
+    int nkv, int hd, int rot_half, int ps, int nslabs, long long slab_stride) {
   const int n = blockIdx.x;
   const float* src = x + (size_t)n * x_stride;
+  auto sums = [&](int at) {
+    float4 v = *reinterpret_cast<const float4*>(src + at);
+    for (int c = 1; c < nslabs; ++c) {
+      const float4 e = *reinterpret_cast<const float4*>(src + (size_t)c * slab_stride + at);
+      v.x += e.x; v.y += e.y; v.z += e.z; v.w += e.w;
+    }
+    return v;
+  };
   const int s = nkv ? slot[n] : -1;
   const size_t page = s >= 0 ? (size_t)(s / ps) : 0, off = s >= 0 ? (size_t)(s % ps) : 0;
   auto add_bias = [&](float4 v, int at) {
@@ -320,8 +330,8 @@ __global__ __launch_bounds__(256) void rope_kv_write_wide_kernel(
       if (s < 0) continue;
       dst = kc + ((page * nkv + (hh - nq)) * ps + off) * hd;
     }
-    const float4 x1 = add_bias(*reinterpret_cast<const float4*>(src + hh * hd + f), hh * hd + f);
-    const float4 x2 = add_bias(*reinterpret_cast<const float4*>(src + hh * hd + f + rot_half), hh * hd + f + rot_half);
+    const float4 x1 = add_bias(sums(hh * hd + f), hh * hd + f);
+    const float4 x2 = add_bias(sums(hh * hd + f + rot_half), hh * hd + f + rot_half);
     const float4 c01 = *reinterpret_cast<const float4*>(cs + (size_t)n * rot_half + f);      // (c0, s0, c1, s1)
     const float4 c23 = *reinterpret_cast<const float4*>(cs + (size_t)n * rot_half + f + 2);
     const float4 lo = {x1.x * c01.x - x2.x * c01.y, x1.y * c01.z - x2.y * c01.w, x1.z * c23.x - x2.z * c23.y,
@@ -342,13 +352,13 @@ __global__ __launch_bounds__(256) void rope_kv_write_wide_kernel(
       if (s < 0) continue;
       dst = kc + ((page * nkv + (hh - nq)) * ps + off) * hd;
     }
-    *reinterpret_cast<uint2*>(dst + d) = pack4(add_bias(*reinterpret_cast<const float4*>(src + hh * hd + d), hh * hd + d));
+    *reinterpret_cast<uint2*>(dst + d) = pack4(add_bias(sums(hh * hd + d), hh * hd + d));
   }
   // values: [page][kv head][channel][slot]
   if (s >= 0) {
     for (int it = threadIdx.x; it < nkv * (hd / 4); it += blockDim.x) {
       const int kvh = it / (hd / 4), d = (it - kvh * (hd / 4)) * 4, at = (nq + nkv + kvh) * hd + d;
-      const float4 v = add_bias(*reinterpret_cast<const float4*>(src + at), at);
+      const float4 v = add_bias(sums(at), at);
       bf16_t* dst = vc + ((page * nkv + kvh) * hd + d) * ps + off;
       dst[0] = f32_to_bf16(v.x);
       dst[(size_t)ps] = f32_to_bf16(v.y);
@@ -359,12 +369,15 @@ __global__ __launch_bounds__(256) void rope_kv_write_wide_kernel(
 }
 
 // cs: null, or float32 [N, rot_half, 2] from qvl_rope_table (then pos, inv_freq and freq_row are not read).
+// nslabs > 1: x is float32 slabs of partial sums, slab_stride elements apart; taken with float32 in,
+// bfloat16 out, cs given and all widths multiples of 4 only (else QVL_ERR_SHAPE).
 extern "C" int qvl_rope_kv_write(const void* x, int x_stride, const void* bias, const void* pos, int pos_stride,
                                  const void* inv_freq, const void* freq_row, const void* cs, const void* slot,
                                  void* q_out, void* kc,
                                  void* vc, int N, int nq, int nkv, int hd, int rot_half, int ps, int in_dtype,
-                                 int dtype, hipStream_t stream) {
+                                 int dtype, int nslabs, long long slab_stride, hipStream_t stream) {
   if (N <= 0) return QVL_OK;
+  if (nslabs < 1 || (nslabs > 1 && (slab_stride < (long long)(nq + 2 * nkv) * hd || slab_stride % 4))) return QVL_ERR_SHAPE;
   if (nq < 0 || nkv < 0 || nq + nkv == 0 || hd <= 0 || rot_half < 0 || 2 * rot_half > hd || ps <= 0)
     return QVL_ERR_SHAPE;
   if (x_stride < (nq + 2 * nkv) * hd) return QVL_ERR_SHAPE;
@@ -373,9 +386,10 @@ extern "C" int qvl_rope_kv_write(const void* x, int x_stride, const void* bias, 
       (((uintptr_t)x | (uintptr_t)bias | (uintptr_t)cs) & 15) == 0 && (((uintptr_t)q_out | (uintptr_t)kc) & 7) == 0) {
     hipLaunchKernelGGL(rope_kv_write_wide_kernel, dim3(N), dim3(256), 0, stream, (const float*)x, x_stride,
                        (const float*)bias, (const float2*)cs, (const int*)slot, (bf16_t*)q_out, (bf16_t*)kc,
-                       (bf16_t*)vc, nq, nkv, hd, rot_half, ps);
+                       (bf16_t*)vc, nq, nkv, hd, rot_half, ps, nslabs, slab_stride);
     return qvl_launch_status();
   }
+  if (nslabs > 1) return QVL_ERR_SHAPE;
   const dim3 grid(N, nq + 2 * nkv);
 #define QVL_ROPE_CASE(ID, OD, TI, T)                                                                               \
   if (in_dtype == ID && dtype == OD) {                                                                             \

@@ -143,7 +143,10 @@ def rope_kv_write(x: torch.Tensor, bias: Optional[torch.Tensor], positions: torc
     ``x`` may be float32 while queries and the cache are bfloat16 (``out_dtype``): the bias is
     added and the rotation done in float32 and each value is rounded once.
 
-    ``x`` is ``[N, (nq + 2 nkv) hd]``: query heads, key heads, value heads.  ``positions`` is
+    ``x`` is ``[N, (nq + 2 nkv) hd]``: query heads, key heads, value heads; or float32
+    ``[slabs, N, (nq + 2 nkv) hd]``, partial sums of a projection cut along its inner size, which are
+    added in slab order before the bias (bfloat16 outputs, ``cs`` given and widths in steps of 4
+    only).  ``positions`` is
     int32 ``[rows, N]``; ``freq_row[f]`` names the row that frequency ``f`` uses (-1: none).
     ``k_cache`` is one layer's ``[pages, nkv, page_size, hd]``, ``v_cache`` its
     ``[pages, nkv, hd, page_size]``.  With ``num_kv_heads == 0`` only queries are rotated.
@@ -153,6 +156,12 @@ def rope_kv_write(x: torch.Tensor, bias: Optional[torch.Tensor], positions: torc
     _dev(x, bias, positions, inv_freq, freq_row, slots, k_cache, v_cache, q_out)
     nq, nkv, hd = int(num_q_heads), int(num_kv_heads), int(head_dim)
     cols = (nq + 2 * nkv) * hd
+    nslabs, slab_stride = 1, 0
+    if x.dim() == 3:
+        _need(x.dtype == torch.float32 and x.is_contiguous() and cs is not None,
+              "slabs of x must be contiguous float32 and come with the table of cosines and sines")
+        nslabs, slab_stride = x.shape[0], x.stride(0)
+        x = x[0]
     n = x.shape[0]
     _need(x.dim() == 2 and x.shape[1] == cols and x.stride(1) == 1, "x must be [N, (nq + 2 nkv) hd]")
     odt = out_dtype or x.dtype
@@ -184,10 +193,11 @@ def rope_kv_write(x: torch.Tensor, bias: Optional[torch.Tensor], positions: torc
               and tuple(cs.shape[1:]) == (rot_half, 2), "cs must be float32 [N, rot/2, 2]")
     fn = _fn("elementwise", "qvl_rope_kv_write",
              [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
-              _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+              _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, ctypes.c_longlong, _c_ptr])
     _check(fn(_ptr(x), x.stride(0), _ptr(bias), _ptr(positions), positions.stride(0), _ptr(inv_freq),
               _ptr(freq_row), _ptr(cs), _ptr(slots), _ptr(q_out), _ptr(k_cache), _ptr(v_cache), n, nq, nkv, hd, rot_half,
-              int(page_size), dtype_code(x.dtype), dtype_code(odt), _stream()), "rope_kv_write")
+              int(page_size), dtype_code(x.dtype), dtype_code(odt), int(nslabs), int(slab_stride), _stream()),
+           "rope_kv_write")
     return q_out
 
 

@@ -111,6 +111,37 @@ def test_rope_kv_write(dtype, nq, nkv, hd, sections, ps):
     assert torch.allclose(qp[..., :2 * half], want.transpose(0, 1), **tol)
 
 
+def test_rope_kv_write_from_slabs():
+    """The projection as slabs of partial sums: the rotation's kernel adds them in order and gives
+    what it gives for their sum."""
+    from qwen25vl_lite_amd.ops import kernels
+    torch.manual_seed(3)
+    n, nq, nkv, hd, ps, pages = 40, 6, 2, 48, 16, 9
+    cols = (nq + 2 * nkv) * hd
+    slabs = torch.randn(3, n, cols).cuda()
+    total = slabs[0] + slabs[1]
+    total = total + slabs[2]
+    bias = torch.randn(cols).cuda()
+    pos = torch.randint(0, 500, (3, n), dtype=torch.int32).cuda()
+    inv_freq = plain_inv_freq(hd, 10000.0).cuda()
+    freq_row = torch.tensor([0] * 8 + [1] * 8 + [2] * 8, dtype=torch.int32).cuda()
+    slots = torch.randperm(pages * ps)[:n].to(torch.int32).cuda()
+    cs = kernels.rope_table(pos, inv_freq, freq_row, n)
+    outs = []
+    for x in (slabs, total):
+        kc = torch.zeros(pages, nkv, ps, hd, dtype=torch.bfloat16).cuda()
+        vc = torch.zeros(pages, nkv, hd, ps, dtype=torch.bfloat16).cuda()
+        q = kernels.rope_kv_write(x, bias, pos, inv_freq, freq_row, slots, kc, vc, nq, nkv, hd, ps,
+                                  out_dtype=torch.bfloat16, cs=cs)
+        outs.append((q, kc, vc))
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+    assert outs[0][0].abs().sum() > 0 and outs[0][1].abs().sum() > 0
+    with pytest.raises(kernels.KernelError):      # slabs are taken with the table in hand only
+        kernels.rope_kv_write(slabs, bias, pos, inv_freq, freq_row, slots, outs[0][1], outs[0][2], nq, nkv, hd, ps,
+                              out_dtype=torch.bfloat16)
+
+
 def _paged(k, v, ps, pages, dtype, seed):
     """Scatter per-request keys/values [nkv, T, hd] into shuffled pages; returns caches and tables."""
     g = torch.Generator().manual_seed(seed)
