@@ -28,8 +28,11 @@ WIDE_WALKS_PER_CU = 3      # the kind of the kernel whose waves carry three colu
 WIDE_BLOCKS_PER_CU = 586   # ... that have this many 32-key blocks to walk between them (150,000 on 256 units)
 TARGET_BLOCKS = None
 FILL_BLOCKS = None
-MIN_KEYS_PER_SPLIT = 1024  # merging the splits (stores, a counter and loads that go through to memory) costs a decode
-                           # step about as much as each wave's walk over four more 32-key blocks: shorter splits lose
+MIN_KEYS_PER_SPLIT = 256   # keys a split has at least
+SPLIT_FROM_KEYS = 768      # shorter contexts are walked by one block: merging splits (stores, a counter and loads that go
+                           # through to memory) costs a decode step about 4.5 us, a block's walk 12.7 us per 1,000 keys
+                           # (one compute unit reads its keys and values at about 80 GB/s); measured at batch 1 and 8:
+                           # 527 keys 11.5 us whole, 11.9 in two splits; 1,024 keys 17.8 whole, 12.0 in four
 MERGE_COUNTERS = 1 << 16   # (tile, kv head) pairs whose splits one launch can merge by itself
 ALONE_KEYS = 4096          # decoded tokens beside prompt portions get a launch of their own from this context on
 WIDE_CT = 3
@@ -97,7 +100,7 @@ def plan_splits(num_tiles: int, nkv: int, max_ctx: int, device=None) -> Tuple[st
     if blocks >= _target_blocks(device):
         return "tile", 1, 0
     want = (_fill_blocks(device) + blocks - 1) // blocks
-    nsplit = max(1, min(want, max_ctx // MIN_KEYS_PER_SPLIT))
+    nsplit = max(1, min(want, max_ctx // MIN_KEYS_PER_SPLIT)) if max_ctx >= SPLIT_FROM_KEYS else 1
     if nsplit == 1:
         return "coop", 1, 0
     # splits begin at a multiple of 32 at or below the first key a tile sees: up to 31 keys more

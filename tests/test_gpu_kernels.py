@@ -307,6 +307,7 @@ def test_mixed_step_with_few_long_decoded_tokens(nq, nkv, hd, window, monkeypatc
     c = _attention_case(torch.bfloat16, nq, nkv, hd, window, lens, qlens)
     monkeypatch.setattr(attention_mfma, "TARGET_BLOCKS", 8)    # the two decoded tokens make 4 blocks, the portions 24 or more
     monkeypatch.setattr(attention_mfma, "MIN_KEYS_PER_SPLIT", 64)
+    monkeypatch.setattr(attention_mfma, "SPLIT_FROM_KEYS", 64)
     monkeypatch.setattr(attention_mfma, "ALONE_KEYS", 128)
     cu = [0]
     for ql in qlens:

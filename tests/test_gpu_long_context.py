@@ -121,8 +121,17 @@ def test_context_of_the_benchmark_through_the_real_dispatch(sharp_d, tokens, dty
     assert len(calls(1, "qvl_attn_mfma_block")) == layers and all(d.get("BLK_CT") == 3 for d in calls(1, "qvl_attn_mfma_block"))
     # single tokens over 8,280 keys: the keys split among blocks at the real limit of keys per split
     per = attention_mfma.MIN_KEYS_PER_SPLIT
-    assert per <= 1024 and attention_mfma.ALONE_KEYS == 4096
-    many = 8280 // per      # as many splits as the limit of keys per split allows: the blocks are few
+    assert per <= 1024 and attention_mfma.ALONE_KEYS == 4096 and attention_mfma.SPLIT_FROM_KEYS <= 4096
+
+    def cut(ctx):
+        """As many splits as the limit of keys per split allows (the blocks are few): their length in
+        whole blocks of 32 keys, and how many of that length cover the context."""
+        most = ctx // per
+        keys = ((ctx + 31 + most - 1) // most + 31) // 32 * 32
+        return (ctx + 31 + keys - 1) // keys, keys
+
+    many = cut(8284)[0]
+    assert many >= 8 and all(cut(c)[0] == many for c in range(8281, 8300))
     for i in range(3, 7):
         assert calls(i, "qvl_attn_mfma_block") == [] and splits(i) == [many] * layers
         assert all(per <= d["keys"] < per + 64 for d in calls(i, "qvl_attn_mfma_coop"))
@@ -132,4 +141,3 @@ def test_context_of_the_benchmark_through_the_real_dispatch(sharp_d, tokens, dty
         assert all(n <= 4 for n in splits(i)[:layers]) and splits(i)[layers:] == [many] * layers
     # both decode: one launch, split by the longer context
     assert calls(9, "qvl_attn_mfma_block") == [] and len(splits(9)) == layers and all(n == many for n in splits(9))
-
