@@ -31,7 +31,7 @@ FILL_BLOCKS = None
 MIN_KEYS_PER_SPLIT = 256   # keys a split has at least
 SPLIT_FROM_KEYS = 768      # shorter contexts are walked by one block: merging splits (stores, a counter and loads that go
                            # through to memory) costs a decode step about 4.5 us, a block's walk 12.7 us per 1,000 keys
-                           # (one compute unit reads its keys and values at about 80 GB/s); measured at batch 1 and 8:
+                           # (one compute unit by itself fetches its keys and values at about 40 GB/s); measured at batch 1 and 8:
                            # 527 keys 11.5 us whole, 11.9 in two splits; 1,024 keys 17.8 whole, 12.0 in four
 MERGE_COUNTERS = 1 << 16   # (tile, kv head) pairs whose splits one launch can merge by itself
 ALONE_KEYS = 4096          # decoded tokens beside prompt portions get a launch of their own from this context on
