@@ -597,7 +597,7 @@ extern "C" int qvl_gemm_resident(const void* x, int ldx, const void* h, int ldh,
   p.rows = 16;
   if (epilogue != EPI_SWIGLU) {
     const long long per_round = 16LL * teams;
-    const long long rounds = (N + per_round - 1) / per_round;
+    const long long rounds = (N + per_round - 1) / per_round;   // (more rounds of shorter tiles lose: a load instruction then carries fewer rows)
     p.rows = (int)((N + rounds * teams - 1) / (rounds * teams));
   }
   p.ntiles = (N + p.rows - 1) / p.rows;
