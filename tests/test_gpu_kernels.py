@@ -513,7 +513,7 @@ def test_gate_up_product_with_the_activation_folded_in(dtype, m, inter, k):
 
 @pytest.mark.parametrize("m, n, k", [(64, 3584, 18944), (17, 509, 352), (33, 130, 200), (48, 1000, 3584), (40, 144, 352),
                                      (64, 37, 8), (25, 4700, 1248), (57, 300, 1256), (1, 3584, 18944), (8, 2048, 11008),
-                                     (16, 37, 4104), (3, 5000, 2056), (49, 8, 2048 * 300 + 8)])
+                                     (16, 37, 4104), (3, 5000, 2056), (49, 8, 2048 * 300 + 8), (4, 512, 29568), (33, 260, 29568)])
 def test_split_product_and_the_norm_that_adds_its_slabs(m, n, k):
     """Up to 64 rows against a weight cut along its inner size: the slabs of partial sums add up to
     the product (inner sizes that are no multiple of 32, row counts that fill no tile, more chunks
