@@ -9,9 +9,7 @@ from typing import Dict, List, Optional, Tuple
 import torch
 
 from ..cache.manager import CacheGroupSpec
-from ..ops import kernels
-from ..ops.linear import linear
-from ..parts.base import (Block, CacheNeed, LayerSlot, Mixer, ParamSpec, Part, ResidualStream, StateNeed,
+from ..parts.base import (Block, CacheNeed, LayerSlot, Mixer, ParamSpec, Part, PartSpec, ResidualStream, StateNeed,
                           StepContext, build_part)
 from .spec import ModelSpec
 
@@ -23,6 +21,11 @@ def _collect(part: Part, prefix: str, out: Dict[str, Tuple[Part, str, ParamSpec]
         out[prefix + local] = (part, local, spec)
     for name, sub in part.sub_parts().items():
         _collect(sub, f"{prefix}{name}.", out)
+
+
+def _prefix_of(name: str) -> str:
+    """``"a.b.weight"`` -> ``"a.b."``: where the tensors of the part behind a named tensor go."""
+    return name[:name.rfind(".") + 1]
 
 
 def _mixers_of(block: Part, prefix: str = "") -> List[Tuple[str, Mixer]]:
@@ -45,8 +48,10 @@ class DecoderModel:
         self.device = torch.device(device)
         self.blocks: List[Block] = [build_part("block", ls.block, dtype, self.device) for ls in spec.layers]
         self.final_norm = build_part("norm", spec.final_norm, dtype, self.device)
-        self.embed: Optional[torch.Tensor] = None
-        self.head: Optional[torch.Tensor] = None
+        sizes = {"vocab_size": spec.vocab_size, "hidden_size": spec.hidden_size}
+        self.embedding = build_part("embedding", spec.embed or PartSpec("token_table", sizes), dtype, self.device)
+        self.head_part = build_part("head", spec.head or PartSpec("linear", sizes), dtype, self.device)
+        self._has_weights = False
 
         # The run list: which cache layer and state every mixer of every entry owns.  The lists
         # below have one element per (run entry, mixer of its block), in run order ("places");
@@ -101,11 +106,14 @@ class DecoderModel:
             self.entry_places.append(places)
 
         self.params: Dict[str, Tuple[Optional[Part], str, ParamSpec]] = {}
-        self.params[spec.embed_name] = (None, "embed", ParamSpec((spec.vocab_size, spec.hidden_size), "table"))
+        _collect(self.embedding, _prefix_of(spec.embed_name), self.params)
         for ls, block in zip(spec.layers, self.blocks):
             _collect(block, ls.prefix, self.params)
         _collect(self.final_norm, spec.final_norm_prefix, self.params)
-        self.params[spec.head_name] = (None, "head", ParamSpec((spec.vocab_size, spec.hidden_size), "matrix"))
+        _collect(self.head_part, _prefix_of(spec.head_name), self.params)
+        for name in (spec.embed_name, spec.head_name):
+            if name not in self.params:
+                raise ValueError(f"the spec names the tensor {name}, which neither end of the model declares")
 
     # ------------------------------------------------------------------ structure
     @property
@@ -113,7 +121,7 @@ class DecoderModel:
         """True if every part may run under HIP graph capture."""
         def safe(part) -> bool:
             return part.graph_safe and all(safe(s) for s in part.sub_parts().values())
-        return all(safe(b) for b in self.blocks) and safe(self.final_norm)
+        return all(safe(b) for b in self.blocks) and safe(self.final_norm) and safe(self.embedding) and safe(self.head_part)
 
     def cache_groups(self) -> List[CacheGroupSpec]:
         return [CacheGroupSpec(need, n) for need, n in zip(self.group_needs, self.group_layers)]
@@ -130,16 +138,22 @@ class DecoderModel:
             groups.setdefault(key, (part, {}))[1][local] = name
         return list(groups.values())
 
-    def load_part(self, part: Optional[Part], tensors: Dict[str, torch.Tensor]) -> None:
-        if part is not None:
-            part.load(tensors)
-        elif "embed" in tensors:
-            self.embed = tensors["embed"]
-        elif "head" in tensors:
-            self.head = tensors["head"]
+    def load_part(self, part: Part, tensors: Dict[str, torch.Tensor]) -> None:
+        part.load(tensors)
+        self._has_weights = True
 
     def tie_head(self) -> None:
-        self.head = self.embed
+        self.head_part.tie(self.embedding)
+
+    @property
+    def embed(self) -> Optional[torch.Tensor]:
+        """The token table (what a tied head shares)."""
+        return self.embedding.table
+
+    @property
+    def head(self) -> Optional[torch.Tensor]:
+        """The built-in head's matrix (None for a head of another kind)."""
+        return getattr(self.head_part, "weight", None)
 
     def make_slots(self, storage, state_tensors: List[Optional[torch.Tensor]]) -> List[LayerSlot]:
         """One slot per run entry.  ``state_tensors`` has one element per place (see
@@ -167,12 +181,12 @@ class DecoderModel:
     def forward(self, step: StepContext, slots: List[LayerSlot]) -> torch.Tensor:
         """Run the step's tokens through the run list; float32 logits ``[M, vocab]`` at
         ``step.logit_rows``."""
-        if self.embed is None or self.head is None:
+        if not self._has_weights:
             raise RuntimeError("the model has no weights yet")
-        stream = ResidualStream(kernels.embed_gather(step.token_ids, self.embed))
+        stream = ResidualStream(self.embedding.forward(step.token_ids, step))
         for entry, slot in zip(self.spec.run, slots):
             stream = self.blocks[entry.layer].forward(stream, step, slot)
         if step.logit_rows.shape[0] == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)
         x = self.final_norm.forward(stream, rows=step.logit_rows)
-        return linear(x, self.head, out_dtype=torch.float32)
+        return self.head_part.forward(x, step)

@@ -50,3 +50,7 @@ class ModelSpec:
     # canonical name -> the name a written model folder stores the tensor under
     store_name: Callable[[str], str] = field(default=lambda name: name)
     eos_token_id: Optional[int] = None
+    # the parts at the two ends; None: a plain token table and a plain linear head of [vocab, hidden].
+    # Their tensors go by ``embed_name`` / ``head_name`` with the last component replaced by the part's own names.
+    embed: Optional[PartSpec] = None
+    head: Optional[PartSpec] = None

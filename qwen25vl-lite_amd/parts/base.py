@@ -33,7 +33,7 @@ import torch
 __all__ = [
     "ParamSpec", "PartSpec", "CacheNeed", "StateNeed", "LayerSlot", "GroupStep", "StepContext", "ResidualStream",
     "Part", "Norm", "Mixer", "FeedForward", "PositionEncoding", "Block", "register_part", "build_part",
-    "known_parts",
+    "known_parts", "Embedding", "Head",
 ]
 
 
@@ -41,10 +41,13 @@ __all__ = [
 class ParamSpec:
     """A tensor a part needs.  ``role`` decides how it is kept on the device:
     ``"matrix"`` and ``"table"`` in the run dtype (bfloat16 or float32), ``"vector"`` in
-    float32 (norm weights, biases: they enter float32 arithmetic), ``"int"`` as int32."""
+    float32 (norm weights, biases: they enter float32 arithmetic), ``"int"`` as int32.
+    ``init`` says how the random-weights mode draws it: ``"normal"`` N(0, std),
+    ``"around_one"`` 1 + N(0, std) (a gain), ``"zeros"``, ``"ones"``."""
 
     shape: Tuple[int, ...]
     role: str = "matrix"
+    init: str = "normal"
 
 
 @dataclass(frozen=True)
@@ -202,8 +205,30 @@ class Block(Part):
         raise NotImplementedError
 
 
+class Embedding(Part):
+    """Token ids to the start of the residual sum.  ``table`` is the tensor a tied head shares."""
+
+    table: Optional[torch.Tensor] = None
+
+    def forward(self, token_ids: torch.Tensor, step: StepContext) -> torch.Tensor:
+        """int32 ``[N]`` -> float32 ``[N, hidden]``."""
+        raise NotImplementedError
+
+
+class Head(Part):
+    """Normalised rows to logits."""
+
+    def forward(self, x, step: StepContext) -> torch.Tensor:
+        """``[rows, hidden]`` -> float32 ``[rows, vocab]``."""
+        raise NotImplementedError
+
+    def tie(self, embedding: Embedding) -> None:
+        """Use the embedding's table instead of a tensor of its own (a model that ties the two)."""
+        raise NotImplementedError
+
+
 _REGISTRY: Dict[str, Dict[str, Callable[..., Part]]] = {
-    "norm": {}, "mixer": {}, "ffn": {}, "position": {}, "block": {},
+    "norm": {}, "mixer": {}, "ffn": {}, "position": {}, "block": {}, "embedding": {}, "head": {},
 }
 
 

@@ -29,7 +29,7 @@ class RMSNorm(Norm):
         self.weight: Optional[torch.Tensor] = None
 
     def param_specs(self) -> Dict[str, ParamSpec]:
-        return {"weight": ParamSpec((self.size,), "vector")}
+        return {"weight": ParamSpec((self.size,), "vector", init="around_one")}
 
     def load(self, tensors):
         self.weight = tensors["weight"]

@@ -3,8 +3,8 @@
 The reference package has no such mode (its tests build a library model under a seed and
 save it, reference tests/conftest.py:76-86).  Here every tensor is drawn from a generator
 seeded by ``(seed, tensor name)``, so a tensor's values do not depend on the order or the
-set of tensors drawn: matrices, tables and biases from N(0, std), norm weights from
-1 + N(0, std).
+set of tensors drawn.  How a tensor is drawn is its part's word (``ParamSpec.init``): N(0, std)
+unless it says otherwise (a norm's weight: 1 + N(0, std)).
 """
 
 from __future__ import annotations
@@ -27,13 +27,17 @@ def _seed_for(seed: int, name: str) -> int:
     return int.from_bytes(digest, "little") & 0x7FFFFFFFFFFFFFFF
 
 
-def _draw(name: str, shape, seed: int, std: float, device, dtype: torch.dtype, role: str = "matrix") -> torch.Tensor:
+def _draw(name: str, shape, seed: int, std: float, device, dtype: torch.dtype, init: str = "normal") -> torch.Tensor:
+    if init in ("zeros", "ones"):
+        return torch.full(tuple(shape), float(init == "ones"), dtype=dtype, device=device)
+    if init not in ("normal", "around_one"):
+        raise ValueError(f"{name}: no rule to draw a tensor with init {init!r}")
     gen = torch.Generator(device=device)
     gen.manual_seed(_seed_for(seed, name))
     t = torch.empty(tuple(shape), dtype=torch.float32, device=device)
     t.normal_(0.0, std, generator=gen)
-    if role == "vector" and name.endswith(".weight"):
-        t += 1.0  # a norm's weight: around one
+    if init == "around_one":
+        t += 1.0
     return t.to(dtype)
 
 
@@ -46,7 +50,7 @@ def random_tensors(model, seed: int, std: float = 0.02, *, device="cpu",
             continue
         if spec.role == "int":
             raise ValueError(f"no rule to draw the integer table {name}")
-        yield name, _draw(name, spec.shape, seed, std, device, dtype or torch.float32, spec.role)
+        yield name, _draw(name, spec.shape, seed, std, device, dtype or torch.float32, spec.init)
 
 
 def write_random_model(config, out_dir: str, seed: int, *, std: float = 0.02,
@@ -86,7 +90,7 @@ def fill_random(model, seed: int, std: float = 0.02) -> None:
                 continue
             spec = expected[name]
             tensors[local] = _draw(name, spec.shape, seed, std, model.device, kept_dtype(spec.role, model.dtype),
-                                   spec.role)
+                                   spec.init)
         if tensors:
             model.load_part(part, tensors)
     if model.spec.tie_word_embeddings:

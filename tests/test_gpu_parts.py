@@ -539,3 +539,76 @@ def test_a_block_with_two_mixers_gets_a_slot_for_each():
         (part.w_out if local == "o_proj.weight" else part.C).zero_()
         assert not torch.allclose(_run(runner, "z", ta, [26]), whole_a, atol=1e-3)
         (part.w_out if local == "o_proj.weight" else part.C).copy_(kept)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_toy_ends_of_the_model(dtype):
+    """The two ends are parts as well: an embedding that scales its rows and a head with a bias and
+    a soft cap, defined here, registered, named in a spec, given random weights and stepped through
+    the runner; the head is tied to the toy embedding's table.  One toy layer sits between them."""
+    from qwen25vl_lite_amd.models import DecoderModel, LayerSpec, ModelSpec, RunEntry
+    from qwen25vl_lite_amd.ops import kernels
+    from qwen25vl_lite_amd.ops.linear import linear
+    from qwen25vl_lite_amd.parts import Embedding, Head, ParamSpec, PartSpec, known_parts, register_part
+    from qwen25vl_lite_amd.weights import fill_random
+
+    class ScaledTable(Embedding):
+        graph_safe = True
+
+        def __init__(self, params, dtype, device):
+            super().__init__(dtype, device)
+            self.vocab, self.hidden, self.scale = params["vocab_size"], params["hidden_size"], float(params["scale"])
+
+        def param_specs(self):
+            return {"weight": ParamSpec((self.vocab, self.hidden), "table")}
+
+        def load(self, tensors):
+            self.table = tensors["weight"]
+
+        def forward(self, token_ids, step):
+            return kernels.embed_gather(token_ids, self.table) * self.scale
+
+    class CappedHead(Head):
+        graph_safe = True
+
+        def __init__(self, params, dtype, device):
+            super().__init__(dtype, device)
+            self.vocab, self.hidden, self.cap = params["vocab_size"], params["hidden_size"], float(params["cap"])
+
+        def param_specs(self):
+            return {"weight": ParamSpec((self.vocab, self.hidden)), "bias": ParamSpec((self.vocab,), "vector")}
+
+        def load(self, tensors):
+            self.bias = tensors["bias"]
+            self.weight = tensors.get("weight", getattr(self, "weight", None))
+
+        def tie(self, embedding):
+            self.weight = embedding.table
+
+        def forward(self, x, step):
+            return self.cap * torch.tanh((linear(x, self.weight, out_dtype=torch.float32) + self.bias) / self.cap)
+
+    if "toy_scaled" not in known_parts("embedding"):
+        register_part("embedding", "toy_scaled", ScaledTable)
+        register_part("head", "toy_capped", CappedHead)
+    hidden, vocab, scale, cap = 64, 97, 8.0, 3.0
+    sizes = {"vocab_size": vocab, "hidden_size": hidden}
+    norm = PartSpec("rms_norm", {"size": hidden, "eps": 1e-5})
+    spec = ModelSpec(hidden_size=hidden, vocab_size=vocab, layers=[], run=[], final_norm=norm, tie_word_embeddings=True,
+                     embed_name="tok.weight", head_name="out.weight", final_norm_prefix="ln_f.",
+                     embed=PartSpec("toy_scaled", dict(sizes, scale=scale)), head=PartSpec("toy_capped", dict(sizes, cap=cap)))
+    model = DecoderModel(spec, dtype, "cuda:0")
+    assert sorted(model.expected_tensors()) == ["ln_f.weight", "out.bias", "out.weight", "tok.weight"]
+    fill_random(model, 5, std=0.3)
+    assert model.head_part.weight is model.embedding.table          # tied: no tensor of its own was drawn
+    runner = _runner(model)
+    tokens = [5, 96, 0, 41, 41, 7]
+    got = _run(runner, "a", tokens, [4, 1, 1])
+    table, g, b = model.embed.float().cpu(), model.final_norm.weight.float().cpu(), model.head_part.bias.float().cpu()
+    h = table[tokens] * scale
+    x = plain_rmsnorm(h, g, 1e-5)
+    if dtype == torch.bfloat16:
+        x = x.bfloat16().float()
+    want = cap * torch.tanh((x @ table.T + b) / cap)
+    tol = dict(atol=1e-4, rtol=1e-4) if dtype == torch.float32 else dict(atol=3e-2, rtol=3e-2)
+    assert torch.allclose(got, want, **tol), (got - want).abs().max()
