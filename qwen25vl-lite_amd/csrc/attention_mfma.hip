@@ -121,6 +121,22 @@ struct BlockRegs {
 
 // CT: column tiles (of 16 columns) a wave carries through the walk; every key block it loads is
 // used for all of them.
+__device__ __forceinline__ void load16_to_lds(const char* base, uint32_t lane_bytes, uint32_t stage, uint32_t offset);
+
+// Keys through LDS (the kernel for few tiles, head size 128).  Read straight into operand
+// registers, a wave's key load covers 16 rows of 64 bytes, 256 bytes apart: a compute unit fetches
+// a third slower that way than with loads that cover 1 KB contiguous (36 against 54 GB/s by
+// itself).  So a wave brings the 32 keys of a block into 8 KB of LDS of its own with eight loads of
+// 1 KB each (straight into LDS, no registers on the way) and reads its operands from there.  Row
+// kappa of the block keeps its 16-byte chunk c at place c ^ f(kappa), f = the row of the
+// matrix-core tile that key has (bits 4, 3, 1, 0 of kappa: the 16 keys one operand read touches
+// have 16 different f), so the 16 lanes of an operand read hit 16 different places of the 256-byte
+// bank period.  The lane that fills place s of row kappa fetches chunk s ^ f(kappa).
+#define K_VIA_LDS (HD == 128)
+struct HalfPages {
+  int page[2], off[2];   // of the two 16-key halves of a block: the same for every lane
+};
+
 template <int CT>
 struct Walk {
   const bf16_t* kc;
@@ -140,6 +156,51 @@ struct Walk {
 #pragma unroll
     for (int b = 0; b < 2; ++b) pg.k[b] = bt[min(krow_key(kb, b), max_key) / ps];
     pg.v = bt[min((kb << 5) + 8 * lg, max_key) / ps];
+  }
+
+  // the table entries of a block's two halves (a page holds a multiple of 16 keys: a half lies in one page)
+  __device__ __forceinline__ void issue_half_pages(int kb, HalfPages& hp) const {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int key = (kb << 5) + 16 * h, idx = min(key, max_key) / ps;
+      hp.page[h] = bt[idx];
+      hp.off[h] = key % ps;
+    }
+  }
+  // this lane's byte offset within a half's 4 KB for the load that fills its place (see above), less the constant part
+  __device__ __forceinline__ uint32_t lds_lane_offset() const {
+    const uint32_t l = threadIdx.x & 63, i = l >> 4;
+    return i * 256u + (((l & 15u) ^ i) << 4);
+  }
+  __device__ __forceinline__ void issue_k_to_lds(const HalfPages& hp, uint32_t stage, uint32_t lane_off) const {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int page = __builtin_amdgcn_readfirstlane(hp.page[h] < 0 ? 0 : hp.page[h]);   // no page: nobody sees these keys
+      const int off = __builtin_amdgcn_readfirstlane(hp.off[h]);
+      const char* from = reinterpret_cast<const char*>(kc + (((size_t)page * nkv + kvh) * ps + (size_t)off) * HD);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t f_fixed = (uint32_t)((h << 3) | ((j >> 1) << 2));
+        load16_to_lds(from + j * 1024, lane_off ^ (f_fixed << 4), stage, (uint32_t)(h * 4 + j) * 1024u);
+      }
+    }
+  }
+  __device__ __forceinline__ void k_from_lds(const char* staged, BlockRegs& rg) const {
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const int kappa = 8 * (r >> 2) + 4 * b + (r & 3);
+      const int f = ((kappa >> 4) << 3) | (((kappa >> 3) & 1) << 2) | (kappa & 3);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        rg.k[b][ks] = *reinterpret_cast<const bf16x8_t*>(staged + kappa * 256 + (((ks * 4 + lg) ^ f) << 4));
+    }
+  }
+  __device__ __forceinline__ void issue_v(int kb, const BlockPages& pg, BlockRegs& rg) const {
+    const int vkey = (kb << 5) + 8 * lg;
+    const int vpage = (pg.v < 0 || vkey > max_key) ? 0 : pg.v;
+    const bf16_t* vbase = vc + (((size_t)vpage * nkv + kvh) * HD) * ps + (size_t)(vkey % ps);
+#pragma unroll
+    for (int dt = 0; dt < NT; ++dt) rg.v[dt] = load8(vbase + (size_t)(dt * 16 + r) * ps);
   }
 
   __device__ __forceinline__ void issue_loads(int kb, const BlockPages& pg, BlockRegs& rg) const {
@@ -343,11 +404,25 @@ struct Walk {
 // Walk the 32-key blocks first, first + stride, ... that overlap keys [key_begin, key_end]
 // (inclusive, absolute) of one tile.  The loads of the next block and the page lookups of the one
 // after are issued before the current block is computed, so a wave always has a block in flight.
+// all but the N loads this wave asked for last have arrived (in LDS or in registers); nothing moves across
+template <int N>
+__device__ __forceinline__ void wait_for_all_but() {
+  static_assert(N == 0 || N == 16, "the counts the walk uses");
+  if (N == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+}
+// every LDS read of this wave has its data: the place it read may be written again
+__device__ __forceinline__ void lds_reads_done() {
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+}
+
 template <int CT>
 __device__ __forceinline__ void attend(const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
                                        const int* __restrict__ bt, int table_width, int nkv, int kvh, int ps,
                                        const bf16x8_t (*qb)[KS], const int* my_lo, const int* my_p, float scale_log2,
-                                       int key_begin, int key_end, int kb_offset, int kb_stride, TileState* st) {
+                                       int key_begin, int key_end, int kb_offset, int kb_stride, TileState* st,
+                                       uint32_t k_stage = 0, const char* k_staged = nullptr, uint32_t k_stage2 = 0,
+                                       const char* k_staged2 = nullptr) {
   const int lane = threadIdx.x & 63;
   Walk<CT> w;
   w.kc = kc; w.vc = vc; w.bt = bt;
@@ -379,6 +454,62 @@ __device__ __forceinline__ void attend(const bf16_t* __restrict__ kc, const bf16
   if (!LIVE(kb)) return;
   BlockPages p0, p1;
   BlockRegs ra, rb;
+  if (K_VIA_LDS && k_staged) {
+    // Keys through two places of 8 KB in LDS that belong to this wave (LDS byte addresses k_stage and
+    // k_stage2); values straight into registers.  Two blocks are on their way at a time: while block kb
+    // is computed, block kb + s is coming in, and block kb + 2 s is asked for as soon as block kb's place
+    // and registers are free.  A block's 16 loads (8 for the values, then 8 for the keys) are the last
+    // thing asked for before the wait for the block before it, so that wait allows exactly 16 loads to
+    // be outstanding (loads finish in the order they were asked for); without a next block it allows none.
+    static_assert(!K_VIA_LDS || NT == 8, "a block's value loads are counted");
+    const uint32_t lane_off = w.lds_lane_offset();
+    HalfPages h0, h1;
+    w.issue_pages(kb, p0);
+    w.issue_half_pages(kb, h0);
+    if (LIVE(kb + s)) {
+      w.issue_pages(kb + s, p1);
+      w.issue_half_pages(kb + s, h1);
+    }
+    w.issue_v(kb, p0, ra);
+    w.issue_k_to_lds(h0, k_stage, lane_off);
+    if (LIVE(kb + s)) {
+      w.issue_v(kb + s, p1, rb);
+      w.issue_k_to_lds(h1, k_stage2, lane_off);
+    }
+    for (;; kb += 2 * s) {
+      if (LIVE(kb + s)) wait_for_all_but<16>();
+      else wait_for_all_but<0>();
+      w.k_from_lds(k_staged, ra);
+      if (LIVE(kb + 2 * s)) {
+        w.issue_pages(kb + 2 * s, p0);
+        w.issue_half_pages(kb + 2 * s, h0);
+      }
+      w.template compute<false>(kb, qb, ra, st);
+      if (!LIVE(kb + s)) break;
+      if (LIVE(kb + 2 * s)) {
+        lds_reads_done();
+        w.issue_v(kb + 2 * s, p0, ra);
+        w.issue_k_to_lds(h0, k_stage, lane_off);
+        wait_for_all_but<16>();
+      } else {
+        wait_for_all_but<0>();
+      }
+      w.k_from_lds(k_staged2, rb);
+      if (LIVE(kb + 3 * s)) {
+        w.issue_pages(kb + 3 * s, p1);
+        w.issue_half_pages(kb + 3 * s, h1);
+      }
+      w.template compute<false>(kb + s, qb, rb, st);
+      if (!LIVE(kb + 2 * s)) break;
+      if (LIVE(kb + 3 * s)) {
+        lds_reads_done();
+        w.issue_v(kb + 3 * s, p1, rb);
+        w.issue_k_to_lds(h1, k_stage2, lane_off);
+      }
+    }
+    lds_reads_done();
+    return;
+  }
   w.issue_pages(kb, p0);
   if (LIVE(kb + s)) w.issue_pages(kb + s, p1);
   w.issue_loads(kb, p0, ra);
@@ -942,6 +1073,7 @@ __global__ __launch_bounds__(64 * COOP_WAVES) void attn_mfma_coop_kernel(
     float* __restrict__ scratch, int* __restrict__ counters, int nq, int nkv, int ps, int window, float scale,
     int nsplit, int keys_per_split) {
   __shared__ __attribute__((aligned(16))) float sm[COOP_WAVES][PART_STRIDE];
+  __shared__ __attribute__((aligned(16))) char second_place[K_VIA_LDS ? COOP_WAVES : 1][K_VIA_LDS ? 32 * HD * 2 : 16];   // of staged keys
   __shared__ int is_last;
   const int tile = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lg = lane >> 4, c = lane & 15;
@@ -961,8 +1093,15 @@ __global__ __launch_bounds__(64 * COOP_WAVES) void attn_mfma_coop_kernel(
   if (first <= last) {
     bf16x8_t qb[1][KS];
     load_q(q, nq, t, qb[0]);
+    // a wave's place in LDS holds its staged keys while it walks, its sums afterwards
+    static_assert(!K_VIA_LDS || PART_STRIDE * 4 >= 32 * HD * 2, "a wave's place in LDS holds a block's keys");
+    const uint32_t k_stage = __builtin_amdgcn_readfirstlane(
+        (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)&sm[wave][0]);
+    const uint32_t k_stage2 = __builtin_amdgcn_readfirstlane(
+        (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)&second_place[K_VIA_LDS ? wave : 0][0]);
     attend<1>(kc, vc, bt + (size_t)r * table_width, table_width, nkv, kvh, ps, qb, &t.my_lo, &t.my_p, scale * LOG2E,
-              first, last, wave, COOP_WAVES, &st);
+              first, last, wave, COOP_WAVES, &st, k_stage, K_VIA_LDS ? reinterpret_cast<const char*>(&sm[wave][0]) : nullptr,
+              k_stage2, &second_place[K_VIA_LDS ? wave : 0][0]);
   }
   // every wave leaves its column sums in LDS: column c, channels dt*16 + 4*lg .. +3, then m and l
   float* mine = &sm[wave][c * PART_COLS];
