@@ -200,7 +200,8 @@ def _attention_case(dtype, nq, nkv, hd, window, lens=(333, 17, 64, 1), qlens=(5,
 
 # other page sizes than 16 (the reference tests 32, reference tests/test_paged_attn_kernel.py:89);
 # 48 is the one where a 32-key block straddles pages at changing places
-PAGE_SIZES = [(14, 2, 128, None, 32), (5, 1, 48, 40, 48), (4, 2, 80, 130, 64), (6, 2, 24, None, 32)]
+PAGE_SIZES = [(14, 2, 128, None, 32), (5, 1, 48, 40, 48), (4, 2, 80, 130, 64), (6, 2, 24, None, 32), (14, 2, 128, 70, 48),
+              (7, 1, 128, None, 64)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
